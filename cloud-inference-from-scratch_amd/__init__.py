@@ -12,7 +12,7 @@ __version__ = "0.1.0"
 _LAZY = {
     "Engine": "engine", "GenerationConfig": "engine", "GenerationResult": "engine",
     "EngineConfig": "config", "build_engine_config": "config", "load_config": "config",
-    "register_architecture": "config", "Qwen2Config": "config",
+    "register_architecture": "config", "Qwen2Config": "config", "PolosunConfig": "config",
 }
 
 

@@ -43,6 +43,8 @@ def register_architecture(
 
 def architecture_of(raw: dict[str, Any]) -> Architecture:
     names = raw.get("architectures") or []
+    if not names and isinstance(raw.get("architecture"), str):  # (some configurations name one, without a list)
+        names = [raw["architecture"]]
     name = names[0] if names else _MODEL_TYPES.get(raw.get("model_type", ""))
     if name is None or name not in ARCHITECTURES:
         raise ConfigError(

@@ -41,6 +41,8 @@ class LayerSpec:
 
     ``names`` maps the block's part roles (``norm1``, ``mixer``, ``norm2``,
     ``feed_forward``) to the sub-prefix of the checkpoint's tensor names.
+    ``options`` are the arrangement's own constants (a factor on the branches, the layer's depth), which
+    the block class reads.
     """
 
     mixer: PartSpec
@@ -49,6 +51,10 @@ class LayerSpec:
     norm2: PartSpec
     block: str = "pre_norm"
     names: tuple[tuple[str, str], ...] = ()
+    options: tuple[tuple[str, Any], ...] = ()
+
+    def option(self, name: str, default: Any = None) -> Any:
+        return dict(self.options).get(name, default)
 
     def name_of(self, role: str) -> str:
         return dict(self.names).get(role, role)

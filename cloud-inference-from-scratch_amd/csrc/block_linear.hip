@@ -1,0 +1,118 @@
+// A block-diagonal product: B independent small products side by side on the column axis, one weight each.
+//
+//   C[m, b, n] = sum_k A[m, b, k] * W[b, n, k] (+ bias[b, n])  (* sigmoid(gate[m, b, n]) if a gate is given)
+//
+//   A    rows lda apart, block b's K numbers start a_block elements after block b - 1's
+//   W    [B, N, K] contiguous;  bias [B, N] or none
+//   C    rows ldc apart, block b's N results start c_block elements after block b - 1's
+//   gate like C, rows ldg apart, blocks g_block apart (in A's type)
+//
+// It serves per-head products (a query folded into a shared latent space and back out of it) and gates made from
+// a channel's own block.  Operands are float32 or bfloat16, sums are float32 fused multiply-adds in one fixed order
+// of k (blocks of 256 summed, then the blocks' sums), so a row's result does not depend on the other rows; the
+// result is float32 or the operands' type.  64 x 64 results per workgroup, slices of 16 k through LDS.
+#include "common.h"
+
+namespace {
+constexpr int TM = 64, TN = 64, TK = 16;
+constexpr int kSlices = 16;
+
+template <typename TA, typename TC>
+__global__ void __launch_bounds__(256)
+block_linear_kernel(const TA* __restrict__ A, long lda, long a_block, const TA* __restrict__ W,
+                    const TA* __restrict__ bias, TC* __restrict__ C, long ldc, long c_block,
+                    const TA* __restrict__ gate, long ldg, long g_block, int M, int N, int K) {
+    __shared__ float a_tile[TK][TM + 4];
+    __shared__ float w_tile[TK][TN + 4];
+    const int b = blockIdx.z;
+    const int m0 = blockIdx.y * TM;
+    const int n0 = blockIdx.x * TN;
+    const int tx = threadIdx.x % 16;
+    const int ty = threadIdx.x / 16;
+    const TA* a_base = A + static_cast<size_t>(b) * a_block;
+    const TA* w_base = W + static_cast<size_t>(b) * N * K;
+    float acc[4][4] = {}, total[4][4] = {};
+    int slice = 0;
+    for (int k0 = 0; k0 < K; k0 += TK) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = threadIdx.x + 256 * r;
+            const int row = idx / TK;
+            const int kk = idx % TK;
+            const int k = k0 + kk;
+            const int m = m0 + row;
+            const int n = n0 + row;
+            a_tile[kk][row] = (m < M && k < K) ? to_float(a_base[static_cast<size_t>(m) * lda + k]) : 0.f;
+            w_tile[kk][row] = (n < N && k < K) ? to_float(w_base[static_cast<size_t>(n) * K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TK; ++kk) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = a_tile[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = w_tile[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        if (++slice == kSlices) {
+            slice = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    total[i][j] += acc[i][j];
+                    acc[i][j] = 0.f;
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float v = total[i][j] + acc[i][j];
+            if (bias) v += to_float(bias[static_cast<size_t>(b) * N + n]);
+            if (gate) {
+                const float g = to_float(gate[static_cast<size_t>(m) * ldg + static_cast<size_t>(b) * g_block + n]);
+                v *= 1.0f / (1.0f + expf(-g));
+            }
+            C[static_cast<size_t>(m) * ldc + static_cast<size_t>(b) * c_block + n] = from_float<TC>(v);
+        }
+    }
+}
+}  // namespace
+
+// dtype: type of A, W, bias and gate; out_f32: the result is float32 whatever the operands' type
+CIE_API int cie_block_linear(void* stream, int dtype, int out_f32, const void* A, long lda, long a_block, const void* W,
+                             const void* bias, void* C, long ldc, long c_block, const void* gate, long ldg, long g_block,
+                             int M, int N, int K, int B) {
+    if (M < 0 || N <= 0 || K <= 0 || B <= 0 || B > 65535 || lda < K || ldc < N) return CIE_BAD_ARGUMENT;
+    if (M == 0) return CIE_OK;
+    const int grid_y = (M + TM - 1) / TM;
+    if (grid_y > 65535) return CIE_BAD_ARGUMENT;
+    dim3 grid((N + TN - 1) / TN, grid_y, B);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CIE_F32)
+        block_linear_kernel<float, float><<<grid, 256, 0, s>>>(
+            static_cast<const float*>(A), lda, a_block, static_cast<const float*>(W), static_cast<const float*>(bias),
+            static_cast<float*>(C), ldc, c_block, static_cast<const float*>(gate), ldg, g_block, M, N, K);
+    else if (dtype == CIE_BF16 && out_f32)
+        block_linear_kernel<bf16_t, float><<<grid, 256, 0, s>>>(
+            static_cast<const bf16_t*>(A), lda, a_block, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias),
+            static_cast<float*>(C), ldc, c_block, static_cast<const bf16_t*>(gate), ldg, g_block, M, N, K);
+    else if (dtype == CIE_BF16)
+        block_linear_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>(
+            static_cast<const bf16_t*>(A), lda, a_block, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias),
+            static_cast<bf16_t*>(C), ldc, c_block, static_cast<const bf16_t*>(gate), ldg, g_block, M, N, K);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

@@ -796,3 +796,253 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
     _run("cie_sample", load_library().cie_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(uniform),
                                                  _ptr(out), _i(rows), _i(vocab), _i(vocab)))
     return out
+
+
+# ---------------------------------------------------------------------------
+# A stream that is averaged over the depth, block-diagonal products, compressed keys, recurrent mixers
+def depth_stream(x: torch.Tensor, branch_a: Optional[torch.Tensor] = None, branch_b: Optional[torch.Tensor] = None,
+                 mult: float = 1.0, history: Optional[torch.Tensor] = None, newest: int = -1,
+                 weights: Optional[torch.Tensor] = None, gains: tuple = (), out_dtype: torch.dtype = torch.float32,
+                 eps: float = 1e-6, want_stream: bool = True):
+    """One layer boundary of a stream whose layers add two parallel branches and whose next input is a weighted
+    average of what the embedding and every layer so far left:
+
+    ``v = x + mult * (branch_a + branch_b)`` (float32; without branches ``v = x``); ``history[newest] = v``;
+    with ``weights`` (float32 [terms]) ``v = sum_j weights[j] * history[j]``; then for every gain ``g`` in
+    ``gains`` (up to two) the rows ``v / sqrt(mean(v^2) + eps) * g`` in ``out_dtype``.
+
+    x float32 [T, H]; branches [T, H] in ``out_dtype``; history float32 [layers + 1, T, H].  Returns
+    ``(stream or None, [normed rows per gain])``; the stream is a new tensor (``want_stream``) unless nothing changed it."""
+    _gpu("x", x, torch.float32, 2)
+    rows, hidden = x.shape
+    if hidden > MAX_NORM_WIDTH:
+        raise ValueError(f"rows of up to {MAX_NORM_WIDTH} numbers, not {hidden}")
+    for name, branch in (("branch_a", branch_a), ("branch_b", branch_b)):
+        if branch is not None:
+            _gpu(name, branch, out_dtype, 2)
+            if branch.shape != x.shape:
+                raise ValueError(f"{name} {tuple(branch.shape)} vs the stream {tuple(x.shape)}")
+    if branch_b is not None and branch_a is None:
+        raise ValueError("a second branch needs a first")
+    terms, stride = 0, 0
+    if history is not None:
+        _gpu("history", history, torch.float32, 3)
+        if tuple(history.shape[1:]) != (rows, hidden) or not -1 <= newest < history.shape[0]:
+            raise ValueError(f"history {tuple(history.shape)} does not hold rows of {tuple(x.shape)} at {newest}")
+        stride = rows * hidden
+    elif newest >= 0:
+        raise ValueError("a place in the history needs the history")
+    if weights is not None:
+        _gpu("weights", weights, torch.float32, 1)
+        terms = weights.shape[0]
+        if history is None or terms > history.shape[0]:
+            raise ValueError(f"{terms} weights for a history of {0 if history is None else history.shape[0]}")
+    if len(gains) > 2 or not eps > 0:
+        raise ValueError("at most two norms, and a positive eps")
+    changed = branch_a is not None or terms > 0
+    stream = torch.empty_like(x) if (want_stream and changed) else None
+    outs = [torch.empty((rows, hidden), dtype=out_dtype, device=x.device) for _ in gains]
+    g = [float(v) for v in gains] + [0.0, 0.0]
+    _run("cie_depth_stream", load_library().cie_depth_stream(
+        _stream(), _i(_code(out_dtype)), _ptr(x), _ptr(branch_a), _ptr(branch_b), _f(mult), _ptr(history), stride,
+        _i(newest), _ptr(weights), _i(terms), _ptr(stream), _ptr(outs[0] if outs else None), _f(g[0]),
+        _ptr(outs[1] if len(outs) > 1 else None), _f(g[1]), _i(rows), _i(hidden), _f(eps)))
+    return (stream if stream is not None else (x if want_stream else None)), outs
+
+
+def block_linear(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 a_block: Optional[int] = None, out: Optional[torch.Tensor] = None, out_offset: int = 0,
+                 c_block: Optional[int] = None, out_dtype: Optional[torch.dtype] = None,
+                 gate: Optional[torch.Tensor] = None, gate_offset: int = 0, a_offset: int = 0) -> torch.Tensor:
+    """A block-diagonal product: ``out[m, b, :] = a[m, b, :] @ weight[b].T (+ bias[b])``, times
+    ``sigmoid(gate[m, b, :])`` if a gate is given.
+
+    ``a`` [M, >= a_offset + (B-1) * a_block + K] with unit inner stride (block b's K numbers start at column
+    ``a_offset + b * a_block``; ``a_block`` defaults to K); ``weight`` [B, N, K]; ``bias`` [B, N].  The result goes to
+    columns ``out_offset + b * c_block`` (``c_block`` defaults to N) of ``out``, a new [M, B * N] tensor of ``out_dtype``
+    (float32 or ``a``'s type) if none is given.  ``gate`` is laid out like the default result from its column
+    ``gate_offset`` on.  float32 sums in one fixed order; float32 operands give a true float32 product."""
+    _gpu("weight", weight, a.dtype, 3)
+    blocks, n, k = weight.shape
+    if not (a.is_cuda and a.dim() == 2 and a.stride(1) == 1 and a.dtype in _CODES):
+        raise ValueError("a must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    a_block = k if a_block is None else a_block
+    m = a.shape[0]
+    if a_offset < 0 or a_block < 0 or a.shape[1] < a_offset + (blocks - 1) * a_block + k:
+        raise ValueError(f"a {tuple(a.shape)} does not hold {blocks} blocks of {k} numbers {a_block} apart from {a_offset}")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), a.shape[1])
+    if bias is not None:
+        _gpu("bias", bias, a.dtype, 2)
+        if tuple(bias.shape) != (blocks, n):
+            raise ValueError(f"bias must be {(blocks, n)}")
+    c_block = n if c_block is None else c_block
+    if out is None:
+        out_dtype = out_dtype or a.dtype
+        out = torch.empty((m, out_offset + (blocks - 1) * c_block + n), dtype=out_dtype, device=a.device)
+    if not (out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == m
+            and out.dtype in (torch.float32, a.dtype)):
+        raise ValueError("out must be a GPU matrix of float32 or a's type with a row per row of a")
+    if out_offset < 0 or c_block < n or out.shape[1] < out_offset + (blocks - 1) * c_block + n:
+        raise ValueError(f"out {tuple(out.shape)} does not hold {blocks} blocks of {n} results {c_block} apart from {out_offset}")
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), out.shape[1])
+    ldg = 0
+    if gate is not None:
+        if not (gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == a.dtype and gate.shape[0] == m
+                and gate.shape[1] >= gate_offset + blocks * n):
+            raise ValueError("the gate must be a matrix of a's type with a row per row of a and a number per result")
+        ldg = gate.stride(0) if m > 1 else max(gate.stride(0), gate.shape[1])
+    esz_a, esz_c = a.element_size(), out.element_size()
+    _run("cie_block_linear", load_library().cie_block_linear(
+        _stream(), _i(_code(a.dtype)), _i(1 if out.dtype == torch.float32 else 0), a.data_ptr() + a_offset * esz_a, lda,
+        a_block, _ptr(weight), _ptr(bias), out.data_ptr() + out_offset * esz_c, ldc, c_block,
+        None if gate is None else gate.data_ptr() + gate_offset * esz_a, ldg, n, _i(m), _i(n), _i(k), _i(blocks)))
+    return out
+
+
+def latent_rows(proj: torch.Tensor, weight: torch.Tensor, heads: int, plain: int, turned: int, latent: int,
+                width: int, eps: float) -> torch.Tensor:
+    """Lay out the rows ``[T, (heads + 2) * width]`` that the rotation-and-cache-write kernel and the attention
+    kernels read for a layer whose keys are compressed (``csrc/latent.hip``): per query head its turned part,
+    room for its folded plain part and zeros; one key ``[turned part | normed latent | zeros]`` and one value
+    ``[zeros | normed latent | zeros]``.  ``proj`` [T, heads * (plain + turned) + latent + turned]."""
+    if not (proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1 and proj.dtype in _CODES):
+        raise ValueError("proj must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens = proj.shape[0]
+    if proj.shape[1] != heads * (plain + turned) + latent + turned or width < turned + latent:
+        raise ValueError(f"proj {tuple(proj.shape)} does not fit {heads} heads of {plain}+{turned} and a latent of {latent}+{turned}")
+    _gpu("weight", weight, dims=1)
+    if weight.shape[0] != latent or weight.dtype not in (proj.dtype, torch.float32):
+        raise ValueError("the latent's norm weight does not fit")
+    rows = torch.empty((tokens, (heads + 2) * width), dtype=proj.dtype, device=proj.device)
+    ldp = proj.stride(0) if tokens > 1 else max(proj.stride(0), proj.shape[1])
+    _run("cie_latent_rows", load_library().cie_latent_rows(
+        _stream(), _i(_code(proj.dtype)), _i(_code(weight.dtype)), _ptr(proj), ldp, _ptr(weight), _ptr(rows), _i(tokens),
+        _i(heads), _i(plain), _i(turned), _i(latent), _i(width), _f(eps)))
+    return rows
+
+
+RETENTION_ROWS = (4, 8, 16, 32)  # rows of a head's memory that one thread keeps in registers
+RETENTION_LDS_FLOATS = 15 * 1024
+
+
+def plan_retention(dim: int, vdim: int) -> tuple[int, int, int]:
+    """(rows per thread, groups of threads, tokens per chunk) of the retention kernel for heads of ``dim`` x ``vdim``."""
+    if vdim > 1024:
+        raise ValueError(f"value heads of up to 1024 numbers, not {vdim}")
+    most_groups = max(1, min(dim, 1024 // vdim))
+    need = -(-dim // most_groups)
+    rows = next((r for r in RETENTION_ROWS if r >= need), None)
+    if rows is None:
+        raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's registers")
+    groups = -(-dim // rows)
+    per_token = 2 * dim + vdim + groups * vdim
+    chunk = min(32, RETENTION_LDS_FLOATS // per_token)
+    if chunk < 1:
+        raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's LDS")
+    return rows, groups, chunk
+
+
+def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optional[torch.Tensor],
+              sin: Optional[torch.Tensor], rot: int, decay: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
+              seq_start: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int, dim: int, vdim: int,
+              eps: float, key_scale: float, longest_position: int) -> torch.Tensor:
+    """Retention over a step's tokens (``csrc/recurrent.hip``).  ``proj`` [T, ...] holds each token's queries, keys
+    (heads x dim), values and gates (heads x vdim) from the columns ``offsets`` on; ``state`` float32
+    [slots, heads, dim, vdim] is read and written at the sequences' slots; cos/sin float32 [positions, rot/2]
+    must reach ``longest_position``.  Returns [T, heads * vdim] in ``proj``'s type."""
+    if not (proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1 and proj.dtype in _CODES):
+        raise ValueError("proj must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens = proj.shape[0]
+    q_off, k_off, v_off, g_off = offsets
+    if max(q_off + heads * dim, k_off + heads * dim, v_off + heads * vdim, g_off + heads * vdim) > proj.shape[1]:
+        raise ValueError(f"proj {tuple(proj.shape)} does not hold the heads at {offsets}")
+    if rot:
+        for name, table in (("cos", cos), ("sin", sin)):
+            _gpu(name, table, torch.float32, 2)
+            if table.shape[1] != rot // 2 or table.shape[0] <= longest_position:
+                raise ValueError(f"{name} {tuple(table.shape)} does not reach position {longest_position} with {rot // 2} pairs")
+    _gpu("decay", decay, torch.float32, 1)
+    _gpu("state", state, torch.float32, 4)
+    if decay.shape[0] != heads or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise ValueError(f"decay {tuple(decay.shape)} / state {tuple(state.shape)} do not fit {heads} heads of {dim} x {vdim}")
+    for name, meta, least in (("seq_slot", seq_slot, sequences), ("seq_start", seq_start, sequences),
+                              ("q_start_loc", q_start_loc, sequences + 1)):
+        _gpu(name, meta, torch.int32, 1)
+        if meta.shape[0] < least:
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
+    rows, groups, chunk = plan_retention(dim, vdim)
+    out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    ldp = proj.stride(0) if tokens > 1 else max(proj.stride(0), proj.shape[1])
+    _run("cie_retention", load_library().cie_retention(
+        _stream(), _i(_code(proj.dtype)), _ptr(proj), ldp, _i(q_off), _i(k_off), _i(v_off), _i(g_off),
+        _ptr(cos if rot else None), _ptr(sin if rot else None), _i(rot), _ptr(decay), _ptr(state), _ptr(seq_slot),
+        _ptr(seq_start), _ptr(q_start_loc), _ptr(out), _i(sequences), _i(heads), _i(dim), _i(vdim), _i(rows), _i(groups),
+        _i(chunk), _f(eps), _f(key_scale)))
+    return out
+
+
+MAX_CONV_TAPS = 16
+
+
+def causal_conv(x: torch.Tensor, taps_w: torch.Tensor, bias: Optional[torch.Tensor], past: torch.Tensor,
+                seq_of_token: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor) -> torch.Tensor:
+    """Per channel, ``out[t] = sum_j taps_w[c, j] * x[t - (taps - 1) + j] + bias[c]`` within each sequence; the inputs
+    before the step come from ``past`` (float32 [slots, max(taps - 1, 1), C], oldest first; zeros for a new
+    sequence).  x [T, C] (a view with unit inner stride), taps_w [C, taps]."""
+    if not (x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.dtype in _CODES):
+        raise ValueError("x must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens, channels = x.shape
+    _gpu("taps_w", taps_w, x.dtype, 2)
+    taps = taps_w.shape[1]
+    if taps_w.shape[0] != channels or not 1 <= taps <= MAX_CONV_TAPS:
+        raise ValueError(f"taps {tuple(taps_w.shape)} for {channels} channels (up to {MAX_CONV_TAPS} taps)")
+    if bias is not None:
+        _gpu("bias", bias, x.dtype, 1)
+        if bias.shape[0] != channels:
+            raise ValueError(f"bias must be [{channels}]")
+    _gpu("past", past, torch.float32, 3)
+    if tuple(past.shape[1:]) != (max(taps - 1, 1), channels):
+        raise ValueError(f"past {tuple(past.shape)} must be [slots, {max(taps - 1, 1)}, {channels}]")
+    for name, meta in (("seq_of_token", seq_of_token), ("seq_slot", seq_slot), ("q_start_loc", q_start_loc)):
+        _gpu(name, meta, torch.int32, 1)
+    if seq_of_token.shape[0] < tokens:
+        raise ValueError("one sequence index per token")
+    out = torch.empty((tokens, channels), dtype=x.dtype, device=x.device)
+    ldx = x.stride(0) if tokens > 1 else max(x.stride(0), channels)
+    _run("cie_causal_conv", load_library().cie_causal_conv(
+        _stream(), _i(_code(x.dtype)), _ptr(x), ldx, _ptr(taps_w), _ptr(bias), _ptr(past), _ptr(seq_of_token),
+        _ptr(seq_slot), _ptr(q_start_loc), _ptr(out), _i(tokens), _i(channels), _i(taps)))
+    return out
+
+
+def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, block_width: int,
+                     rate: torch.Tensor, state: torch.Tensor, past: torch.Tensor, seq_slot: torch.Tensor,
+                     q_start_loc: torch.Tensor, sequences: int, taps: int) -> torch.Tensor:
+    """The gated linear recurrence of ``csrc/recurrent.hip`` over a step's tokens: per channel
+    ``a = exp(rate * sigmoid(r))``, ``S = a * S + sqrt(1 - a^2) * sigmoid(i) * u``, ``out = S * gelu_tanh(y_pre)``,
+    with r and i from ``gates`` (float32 [T, 2C], per block of ``block_width`` channels its r then its i).  ``state``
+    float32 [slots, C]; ``past`` float32 [slots, max(taps - 1, 1), C] is moved on with the step's ``x_in``."""
+    tokens, channels = u.shape
+    for name, t in (("y_pre", y_pre), ("x_in", x_in)):
+        if not (t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.dtype == u.dtype and tuple(t.shape) == (tokens, channels)):
+            raise ValueError(f"{name} must be a [{tokens}, {channels}] view of u's type with unit inner stride")
+    _gpu("u", u, dims=2)
+    _gpu("gates", gates, torch.float32, 2)
+    _gpu("rate", rate, torch.float32, 1)
+    _gpu("state", state, torch.float32, 2)
+    _gpu("past", past, torch.float32, 3)
+    if (tuple(gates.shape) != (tokens, 2 * channels) or rate.shape[0] != channels or state.shape[1] != channels
+            or tuple(past.shape[1:]) != (max(taps - 1, 1), channels) or channels % block_width
+            or not 1 <= taps <= MAX_CONV_TAPS):
+        raise ValueError("gates, rate, state or past do not fit the channels")
+    for name, meta, least in (("seq_slot", seq_slot, sequences), ("q_start_loc", q_start_loc, sequences + 1)):
+        _gpu(name, meta, torch.int32, 1)
+        if meta.shape[0] < least:
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
+    out = torch.empty((tokens, channels), dtype=u.dtype, device=u.device)
+    ld = lambda t: t.stride(0) if tokens > 1 else max(t.stride(0), channels)
+    _run("cie_gated_recurrence", load_library().cie_gated_recurrence(
+        _stream(), _i(_code(u.dtype)), _ptr(y_pre), ld(y_pre), _ptr(x_in), ld(x_in), _ptr(u), _ptr(gates),
+        _i(block_width), _ptr(rate), _ptr(state), _ptr(past), _ptr(seq_slot), _ptr(q_start_loc), _ptr(out),
+        _i(sequences), _i(channels), _i(taps)))
+    return out

@@ -7,15 +7,20 @@ returns the feed-forward output as ``pending`` instead of adding it.  A part
 that can add its output into the residual itself (the fused decode products do)
 returns a ``RowSumsq`` or an ``Added`` instead, and the next norm then runs its
 cheaper form or rides along with the product behind it (``parts/linear.py``).
+
+``ParallelDepthBlock``: both branches read the same stream, and the next layer reads a weighted average of what
+the embedding and all layers so far left (below).
 """
 
 from __future__ import annotations
 
-from typing import Optional
+from dataclasses import dataclass, replace
+from typing import Any, Optional
 
 import torch
 
 from ..config.specs import LayerSpec
+from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
 from .linear import Added, RawRows, RowSumsq
@@ -87,3 +92,112 @@ def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, rows=No
 
 
 register_part("block", "pre_norm", PreNormBlock)
+
+
+@dataclass
+class NormedRows:
+    """Stands where a pending branch would: the stream is whole, and these are its rows under the two norms of the
+    block that comes next (a block whose last kernel makes them hands them on; ``second`` is ``None`` where that
+    block has no feed-forward)."""
+
+    first: torch.Tensor
+    second: Optional[torch.Tensor]
+    owner: Any  # the block they were made for
+
+
+class ParallelDepthBlock:
+    """A layer whose two branches read the same stream, and whose successor reads an average over the depth:
+
+        X_new = x + mult * (mixer(norm1(x)) + feed_forward(norm2(x)))
+        x     = sum_j average[j] * X_j        j = 0 .. depth + 1
+
+    with X_0 the embedding's rows and X_(i+1) what layer i left (``X_new``), all float32.  The model keeps the
+    ``X_j`` of a step (``keeps_history``) and hands them to every call.  ``average`` is the checkpoint tensor
+    ``<layer>dwa`` with ``depth + 2`` numbers; ``mult`` and ``depth`` are the layer's options.  One kernel adds the
+    branches, stores X_new, averages and makes the two norms of the block that follows (``link_next``); the first
+    block of a model makes its own norms.  A layer without feed-forward has no second norm; a checkpoint that holds
+    one all the same is accepted."""
+
+    keeps_history = True
+
+    def __init__(self, spec: LayerSpec) -> None:
+        self.spec = spec
+        self.mult = float(spec.option("mult", 1.0))
+        self.depth = int(spec.option("depth", 0))
+        self.average_name = str(spec.option("average_name", "dwa"))
+        self.norm1 = build_part("norm", spec.norm1)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.feed_forward = build_part("feed_forward", spec.feed_forward)
+        self.has_feed_forward = spec.feed_forward.kind != "none"
+        self.norm2 = build_part("norm", spec.norm2)
+        self.next_block: Any = None
+        for norm in (self.norm1, self.norm2):
+            if not hasattr(norm, "gain"):
+                raise ValueError("this arrangement takes norms with one gain (rms_norm_scalar)")
+
+    def link_next(self, block: Any) -> None:
+        """The block that runs after this one (``None``: the last); its norms ride in this block's last kernel."""
+        self.next_block = block if isinstance(block, ParallelDepthBlock) else None
+
+    def _parts(self):
+        parts = [("norm1", self.norm1), ("mixer", self.mixer)]
+        if self.has_feed_forward:
+            parts += [("norm2", self.norm2), ("feed_forward", self.feed_forward)]
+        return parts
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        out: dict[str, TensorSpec] = {}
+        for role, part in self._parts():
+            out.update(part.expected_tensors(f"{prefix}{self.spec.name_of(role)}."))
+        if not self.has_feed_forward:
+            for name, spec in self.norm2.expected_tensors(f"{prefix}{self.spec.name_of('norm2')}.").items():
+                out[name] = replace(spec, optional=True)
+        out[prefix + self.average_name] = TensorSpec((self.depth + 2,), init="norm", keeps_float32=True)
+        return out
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        self.dtype = dtype
+        for role, part in self._parts():
+            part.bind(tensors, f"{prefix}{self.spec.name_of(role)}.", dtype, device)
+        self.average = tensors[prefix + self.average_name].float().contiguous()
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for _, part in self._parts())
+
+    def warm_up(self, rows: int) -> None:
+        for _, part in self._parts():
+            warm = getattr(part, "warm_up", None)
+            if warm is not None:
+                warm(rows)
+
+    def gains(self) -> tuple:
+        return (self.norm1.gain, self.norm2.gain) if self.has_feed_forward else (self.norm1.gain,)
+
+    def forward(self, residual: torch.Tensor, pending, batch, view, writes: bool = True, history=None):
+        if history is None:
+            raise ValueError("a layer that averages over the depth needs the model to keep what every layer left")
+        if isinstance(pending, NormedRows) and pending.owner is self:
+            first, second = pending.first, pending.second
+        else:
+            if pending is not None and not isinstance(pending, (Added, NormedRows)):
+                raise ValueError("a branch that is still to be added cannot be handed to this arrangement")
+            _, normed = ops.depth_stream(residual, gains=self.gains(), out_dtype=self.dtype, eps=self.norm1.eps,
+                                         want_stream=False)
+            first, second = normed[0], normed[1] if len(normed) > 1 else None
+        mixed = self.mixer.forward(first, batch, view, writes)
+        fed = self.feed_forward.forward(second) if self.has_feed_forward else None
+        follower = self.next_block
+        stream, normed = ops.depth_stream(
+            residual, mixed, fed, mult=self.mult, history=history, newest=self.depth + 1, weights=self.average,
+            gains=follower.gains() if follower is not None else (), out_dtype=self.dtype,
+            eps=follower.norm1.eps if follower is not None else self.norm1.eps)
+        if follower is None:
+            return stream, None
+        return stream, NormedRows(normed[0], normed[1] if len(normed) > 1 else None, follower)
+
+
+register_part("block", "parallel_depth_average", ParallelDepthBlock)

@@ -19,25 +19,27 @@ class GatedMLP(Part):
     graph_safe = True
     adds_to_residual = True
     takes_scaled_rows = True  # its first product applies the scale of rows that come without it
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
         if activation != "silu":
             raise ValueError(f"gated feed-forward runs silu only, got {activation!r}")
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        self.names = tuple(names)  # what the checkpoint calls the gate, up and down weights under the part's prefix
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        gate, up, down = self.names
         return {
-            prefix + "gate_proj.weight": TensorSpec((self.intermediate_size, self.hidden_size)),
-            prefix + "up_proj.weight": TensorSpec((self.intermediate_size, self.hidden_size)),
-            prefix + "down_proj.weight": TensorSpec((self.hidden_size, self.intermediate_size)),
+            prefix + gate: TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + up: TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + down: TensorSpec((self.hidden_size, self.intermediate_size)),
         }
 
     def bind(self, tensors, prefix, dtype, device) -> None:
         super().bind(tensors, prefix, dtype, device)
-        self.w_gate_up = torch.cat(
-            [tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]], dim=0
-        ).contiguous()
-        self.w_down = tensors[prefix + "down_proj.weight"].contiguous()
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[prefix + gate], tensors[prefix + up]], dim=0).contiguous()
+        self.w_down = tensors[prefix + down].contiguous()
 
     def warm_up(self, rows: int) -> None:
         self.forward(torch.zeros((rows, self.hidden_size), dtype=self.w_down.dtype, device=self.w_down.device))
@@ -46,4 +48,17 @@ class GatedMLP(Part):
         return linear(linear(x, self.w_gate_up, epilogue="silu"), self.w_down, into=residual)
 
 
+class NoFeedForward(Part):
+    """A layer without a feed-forward: no tensors, and ``forward`` gives nothing to add."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int = 0) -> None:
+        self.hidden_size = hidden_size
+
+    def forward(self, x, residual: Optional[torch.Tensor] = None):
+        return None
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "none", NoFeedForward)

@@ -50,6 +50,15 @@ class DecoderModel:
         self.final_norm = build_part("norm", spec.final_norm)
         self.embedding: torch.Tensor | None = None
         self.head: torch.Tensor | None = None
+        # blocks that read what every earlier layer left (``keeps_history``) are handed a float32 tensor
+        # [calls + 1, tokens, hidden] of the step: row 0 the embedding's rows, row i + 1 what call i left
+        self.keeps_history = any(getattr(block, "keeps_history", False) for block in self.blocks)
+        calls = [self.blocks[call.layer] for call in spec.order]
+        if len(set(map(id, calls))) == len(calls):  # (a layer that runs twice has no single successor)
+            for block, follower in zip(calls, calls[1:] + [None]):
+                link = getattr(block, "link_next", None)
+                if link is not None:
+                    link(follower)
 
     def expected_tensors(self) -> dict[str, TensorSpec]:
         return _expected(self.spec, self.blocks, self.final_norm)
@@ -115,11 +124,17 @@ class DecoderModel:
 
     def forward(self, batch, cache) -> torch.Tensor:
         """Run the step's tokens; float32 logits ``[len(logit_rows), vocab]``."""
-        residual = ops.embed(self.embedding, batch.token_ids, feed=batch.token_feed, pool=batch.token_pool)
+        history = None
+        if self.keeps_history:
+            history = torch.empty((len(self.spec.order) + 1, batch.token_ids.shape[0], self.embedding.shape[1]),
+                                  dtype=torch.float32, device=self.embedding.device)
+        residual = ops.embed(self.embedding, batch.token_ids, feed=batch.token_feed, pool=batch.token_pool,
+                             out=history[0] if history is not None else None)
         pending = None
         for call in self.spec.order:
-            residual, pending = self.blocks[call.layer].forward(
-                residual, pending, batch, cache.view(call.cache), call.writes)
+            block = self.blocks[call.layer]
+            extra = {"history": history} if getattr(block, "keeps_history", False) else {}
+            residual, pending = block.forward(residual, pending, batch, cache.view(call.cache), call.writes, **extra)
         if batch.logit_rows.shape[0] == 0:  # a step of prompt portions that end before their prompts do
             return torch.empty((0, self.head.shape[0]), dtype=torch.float32, device=residual.device)
         selected = normalise(self.final_norm, residual, pending, self.dtype, rows=batch.logit_rows)

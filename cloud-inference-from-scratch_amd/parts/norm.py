@@ -57,4 +57,37 @@ class RMSNorm(Part):
         return ops.add_rmsnorm(residual, branch, self.weight, self.eps, out_dtype, rows=rows)
 
 
+class ScalarRMSNorm(Part):
+    """RMS norm with one gain for all coordinates: ``x * rsqrt(mean(x^2) + eps) * g``.  The checkpoint holds ``g``
+    as a tensor without dimensions whose name is the norm's own (the prefix it is bound under, less the dot).
+    Statistics and scaling are float32.  ``gain`` is what a kernel that makes this norm beside other work
+    (``ops.depth_stream``) is given; ``forward`` serves everyone else through the vector norm's kernel."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float) -> None:
+        if size <= 0 or not eps > 0:
+            raise ValueError(f"a norm needs a positive size and eps, got {size}, {eps}")
+        if size > ops.MAX_NORM_WIDTH:
+            raise ValueError(f"the norm kernels take rows of up to {ops.MAX_NORM_WIDTH} numbers, not {size}")
+        self.size = size
+        self.eps = eps
+        self.gain = 1.0
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {prefix.rstrip("."): TensorSpec((), init="norm", keeps_float32=True)}
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.gain = float(tensors[prefix.rstrip(".")].float().item())
+        self.weight_f32 = torch.full((self.size,), self.gain, dtype=torch.float32, device=device)
+
+    def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(branch, (Added, RowSumsq)):
+            branch = None
+        return ops.add_rmsnorm(residual, branch, self.weight_f32, self.eps, out_dtype, rows=rows)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "rms_norm_scalar", ScalarRMSNorm)

@@ -1,0 +1,144 @@
+"""Mixers with a state of fixed size per request (``FixedState`` cache units) instead of a growing cache.
+
+``Retention``: linear attention with a fixed decay per head and neither softmax nor denominator.  With
+``q, k`` (heads x dim) turned by the position and ``k`` scaled by ``dim^-1/2`` after the turn, ``v`` (heads x vdim):
+``S_t = decay_h S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t``; each head's ``o_t`` is divided by its root mean square
+(no weight), the heads are concatenated, multiplied by ``silu(W_g x)`` and projected.  The state ``S`` [heads, dim,
+vdim] is float32.
+
+``GatedLinearRecurrence``: two branches of ``width`` channels, ``y = gelu_tanh(W_y x + b_y)`` and
+``u = conv(W_x x + b_x)`` (a causal convolution over each channel's last ``taps`` inputs); per block of channels
+``r = sigmoid(A_b u_b + a_b)``, ``i = sigmoid(B_b u_b + b_b)``; ``a = exp(-8 r softplus(lambda))``,
+``S_t = a S_(t-1) + sqrt(1 - a^2) i u_t``; the output is ``W_o (S_t y_t)``.  Its state is ``S`` [width] and the
+convolution's last ``taps - 1`` inputs, both float32.
+
+Both read their sequences' slots and lengths from the step's device tensors (``csrc/recurrent.hip``), run a step's
+tokens in order from the state the earlier steps left and write it back, so a prompt may be cut anywhere.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..cache.manager import FixedState
+from ..config.specs import PartSpec
+from ..kernels import ops
+from ..weights.tensors import TensorSpec
+from .base import Part, build_part, register_part
+from .linear import linear
+
+
+class Retention(Part):
+    graph_safe = False  # (the rotation tables of a model without a longest position grow with the step's context)
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay: tuple, eps: float,
+                 position: PartSpec) -> None:
+        if min(hidden_size, num_heads, head_dim, value_dim) < 1:
+            raise ValueError("sizes must be positive")
+        decay = tuple(float(d) for d in decay)
+        if len(decay) != num_heads:
+            raise ValueError(f"one decay per head: {len(decay)} for {num_heads} heads")
+        if not eps > 0:
+            raise ValueError("eps must be positive")
+        ops.plan_retention(head_dim, value_dim)  # (refuses heads the kernel has no room for)
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.value_dim = value_dim
+        self.decay_values = decay
+        self.eps = float(eps)
+        self.position = build_part("position", position)
+
+    def cache_need(self) -> FixedState:
+        return FixedState((self.num_heads, self.head_dim, self.value_dim))
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, d, v, hidden = self.num_heads, self.head_dim, self.value_dim, self.hidden_size
+        return {
+            prefix + "q": TensorSpec((h * d, hidden)),
+            prefix + "k": TensorSpec((h * d, hidden)),
+            prefix + "v": TensorSpec((h * v, hidden)),
+            prefix + "g": TensorSpec((h * v, hidden)),
+            prefix + "o": TensorSpec((hidden, h * v)),
+        }
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.w_in = torch.cat([tensors[prefix + n] for n in ("q", "k", "v", "g")], dim=0).contiguous()
+        self.w_o = tensors[prefix + "o"].contiguous()
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=device)
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if not writes:
+            raise ValueError("a recurrent mixer moves its state on whenever it runs")
+        h, d, v = self.num_heads, self.head_dim, self.value_dim
+        rot = self.position.rotary_dim if self.position.rotates else 0
+        if rot and batch.max_context > self.position.max_position:
+            raise ValueError(f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}")
+        cos, sin = self.position.tables(x.device, batch.max_context) if rot else (None, None)
+        proj = linear(x, self.w_in)
+        out = ops.retention(proj, (0, h * d, 2 * h * d, 2 * h * d + h * v), cos, sin, rot, self.decay, view.state,
+                            batch.seq_slot, batch.seq_start, batch.q_start_loc, batch.sequences, h, d, v, self.eps,
+                            d ** -0.5, batch.max_context - 1)
+        return linear(out, self.w_o)
+
+
+class GatedLinearRecurrence(Part):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, width: int, blocks: int, taps: int) -> None:
+        if min(hidden_size, width, blocks, taps) < 1 or width % blocks:
+            raise ValueError(f"{width} channels in {blocks} equal blocks, {taps} taps: sizes must be positive and divide")
+        if taps > ops.MAX_CONV_TAPS:
+            raise ValueError(f"the convolution takes up to {ops.MAX_CONV_TAPS} taps, not {taps}")
+        self.hidden_size = hidden_size
+        self.width = width
+        self.blocks = blocks
+        self.taps = taps
+
+    def cache_need(self) -> tuple:
+        return (FixedState((self.width,)), FixedState((max(self.taps - 1, 1), self.width)))
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        w, b, hidden = self.width, self.blocks, self.hidden_size
+        per = w // b
+        return {
+            prefix + "y": TensorSpec((w, hidden)), prefix + "y.b": TensorSpec((w,)),
+            prefix + "x": TensorSpec((w, hidden)), prefix + "x.b": TensorSpec((w,)),
+            prefix + "conv": TensorSpec((w, self.taps)), prefix + "conv.b": TensorSpec((w,)),
+            prefix + "ra": TensorSpec((b, per, per)), prefix + "ra.b": TensorSpec((b, per)),
+            prefix + "ri": TensorSpec((b, per, per)), prefix + "ri.b": TensorSpec((b, per)),
+            prefix + "lam": TensorSpec((w,)),
+            prefix + "o": TensorSpec((hidden, w)),
+        }
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.w_in = torch.cat([tensors[prefix + "y"], tensors[prefix + "x"]], dim=0).contiguous()
+        self.b_in = torch.cat([tensors[prefix + "y.b"], tensors[prefix + "x.b"]], dim=0).contiguous()
+        self.conv_w = tensors[prefix + "conv"].contiguous()
+        self.conv_b = tensors[prefix + "conv.b"].contiguous()
+        # per block the weights of its r gate over those of its i gate: one block-diagonal product makes both
+        self.w_gates = torch.cat([tensors[prefix + "ra"], tensors[prefix + "ri"]], dim=1).contiguous()
+        self.b_gates = torch.cat([tensors[prefix + "ra.b"], tensors[prefix + "ri.b"]], dim=1).contiguous()
+        self.rate = (-8.0 * torch.nn.functional.softplus(tensors[prefix + "lam"].float())).contiguous()
+        self.w_o = tensors[prefix + "o"].contiguous()
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if not writes:
+            raise ValueError("a recurrent mixer moves its state on whenever it runs")
+        state, past = view[0].state, view[1].state
+        w = self.width
+        proj = linear(x, self.w_in, self.b_in)
+        y_pre, x_in = proj[:, :w], proj[:, w:]
+        u = ops.causal_conv(x_in, self.conv_w, self.conv_b, past, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
+        gates = ops.block_linear(u, self.w_gates, self.b_gates, out_dtype=torch.float32)
+        out = ops.gated_recurrence(y_pre, x_in, u, gates, w // self.blocks, self.rate, state, past, batch.seq_slot,
+                                   batch.q_start_loc, batch.sequences, self.taps)
+        return linear(out, self.w_o)
+
+
+register_part("mixer", "retention", Retention)
+register_part("mixer", "gated_linear_recurrence", GatedLinearRecurrence)

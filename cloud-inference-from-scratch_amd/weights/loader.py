@@ -94,7 +94,7 @@ class SafetensorsSource:
 
         tied_optional = dict(tied_optional or {})
         index = self._index()
-        missing = sorted(set(expected) - set(index))
+        missing = sorted(name for name in set(expected) - set(index) if not expected[name].optional)
         unexpected = sorted(set(index) - set(expected) - set(tied_optional))
         wrong = [
             f"{name}: expected {tuple(spec.shape)}, got {index[name][1]}"
@@ -125,7 +125,7 @@ class SafetensorsSource:
             tensor = stored(name)
             return tensor.to(_target_dtype(expected[name], tensor.dtype, target)).to(device)
 
-        return TensorsOnDemand(expected, make)
+        return TensorsOnDemand([name for name in expected if name in index], make)
 
     def load(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
              tied_optional: Mapping[str, str] | None = None) -> dict[str, torch.Tensor]:

@@ -11,9 +11,11 @@ class TensorSpec:
     it: ``"normal"`` is N(0, std), ``"norm"`` is 1 + N(0, std).  ``kind`` is
     ``"float"`` (runs in the engine's dtype) or ``"int"`` (kept as int32).
     ``keeps_float32``: a small vector (norm weight) that stays in 32-bit when the
-    file stores it so, whatever the engine's dtype."""
+    file stores it so, whatever the engine's dtype.  ``optional``: a tensor that a checkpoint may hold although
+    this model does not read it; it is neither missed nor called unexpected."""
 
     shape: tuple[int, ...]
     init: str = "normal"
     kind: str = "float"
     keeps_float32: bool = False
+    optional: bool = False
