@@ -51,7 +51,15 @@ class PolosunConfig:
         for key in ("vocab", "width"):
             _positive_int(raw, key, "config")
         config = cls(copy.deepcopy(raw))
-        config.model_spec()  # (everything else is checked where it is read)
+        spec = config.model_spec()  # (everything else is checked where it is read ...
+        from ..parts.model import expected_tensors  # ... or by the parts themselves, built once here)
+
+        try:
+            expected_tensors(spec)
+        except (KeyError, TypeError, ValueError) as error:
+            if isinstance(error, ConfigError):
+                raise
+            raise ConfigError(f"config: {error}") from error
         return config
 
     def to_hf_config(self) -> dict[str, Any]:
