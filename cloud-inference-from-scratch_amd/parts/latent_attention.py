@@ -29,8 +29,14 @@ from .base import Part, build_part, register_part
 from .linear import linear
 
 
+def positions_bound(batch) -> int:
+    """Positions a step's rotation tables have to reach: its longest context, or, for a step that is captured and
+    replayed with other contexts, the bound it was captured for."""
+    return batch.static_plan.max_keys if batch.static_plan is not None else batch.max_context
+
+
 class LatentAttention(Part):
-    graph_safe = False  # (the rotation tables of a model without a longest position grow with the step's context)
+    graph_safe = True  # (a captured step's rotation tables reach the bound the step was captured for)
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int,
                  scale: float, eps: float, position: PartSpec) -> None:
@@ -94,7 +100,7 @@ class LatentAttention(Part):
         rows = ops.latent_rows(proj[:, : queries + c + r], self.latent_weight, h, p, r, c, width, self.eps)
         ops.block_linear(proj, self.w_fold, a_block=p + r, out=rows, out_offset=r, c_block=width)
         turns = bool(r) and self.position.rotates
-        cos, sin = self.position.tables(x.device, batch.max_context)
+        cos, sin = self.position.tables(x.device, positions_bound(batch))
         ops.rope_kv_write(rows, cos, sin, batch.positions, batch.seq_of_token, batch.seq_slot, view.block_table,
                           view.k_pool, view.v_pool, h, 1, width, rotate=turns, write_kv=writes,
                           rotary_dim=r if turns else None)

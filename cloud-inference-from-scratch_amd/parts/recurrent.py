@@ -27,11 +27,12 @@ from ..config.specs import PartSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, build_part, register_part
+from .latent_attention import positions_bound
 from .linear import linear
 
 
 class Retention(Part):
-    graph_safe = False  # (the rotation tables of a model without a longest position grow with the step's context)
+    graph_safe = True  # (a captured step's rotation tables reach the bound the step was captured for)
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay: tuple, eps: float,
                  position: PartSpec) -> None:
@@ -77,11 +78,12 @@ class Retention(Part):
         rot = self.position.rotary_dim if self.position.rotates else 0
         if rot and batch.max_context > self.position.max_position:
             raise ValueError(f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}")
-        cos, sin = self.position.tables(x.device, batch.max_context) if rot else (None, None)
+        bound = positions_bound(batch)
+        cos, sin = self.position.tables(x.device, bound) if rot else (None, None)
         proj = linear(x, self.w_in)
         out = ops.retention(proj, (0, h * d, 2 * h * d, 2 * h * d + h * v), cos, sin, rot, self.decay, view.state,
                             batch.seq_slot, batch.seq_start, batch.q_start_loc, batch.sequences, h, d, v, self.eps,
-                            d ** -0.5, batch.max_context - 1)
+                            d ** -0.5, bound - 1)
         return linear(out, self.w_o)
 
 

@@ -108,7 +108,7 @@ class Fixed:
         return {name: self.tensors[name].to(target).to(device) for name in expected if name in self.tensors}
 
 
-def make_runner(raw, weights, dtype, kv_tokens, page_size=16, max_running=4, max_model_len=None):
+def make_runner(raw, weights, dtype, kv_tokens, page_size=16, max_running=4, max_model_len=None, graph_decode=False):
     from cie_amd.config import build_engine_config, config_from_dict
     from cie_amd.engine import Runner
     from cie_amd.engine.loading import build_model
@@ -116,7 +116,7 @@ def make_runner(raw, weights, dtype, kv_tokens, page_size=16, max_running=4, max
     model = build_model(config_from_dict(raw))
     model.load(Fixed(weights), dtype, "cuda:0")
     engine_config = build_engine_config(dtype=dtype, page_size=page_size, kv_tokens=kv_tokens, max_running=max_running,
-                                        max_model_len=max_model_len or kv_tokens, prefix_cache_pages=0, graph_decode=False)
+                                        max_model_len=max_model_len or kv_tokens, prefix_cache_pages=0, graph_decode=graph_decode)
     return Runner(model, engine_config, "cuda:0")
 
 

@@ -107,6 +107,23 @@ def test_logits_do_not_depend_on_cutting_or_batching(models, name, schedule, dty
     run_and_compare(raw, weights, requests, SCHEDULES[schedule](requests), dtype, plain)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(pu.SMALL))
+def test_captured_steps_give_the_same_logits(models, name, dtype):
+    """Steps of single tokens replay captured graphs (and short mixed steps theirs, from the second time a shape
+    comes), with uncaptured steps between the replays: every replay is checked against the plain logits, and states
+    move on once per token although a capture runs the kernels on rows of padding."""
+    raw, weights, requests, plain = models[name]
+    steps = replay_util.fixed_portions(requests, portion=8, live=3, decode_tail=14)
+    pool = max(replay_util.max_live_tokens(steps, page=16), 16)
+    runner = pu.make_runner(raw, weights, dtype, pool, 16, 4, graph_decode=True)
+    assert runner.graphs is not None, "the model's parts all say that they may be captured"
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    worst, rms = pu.spread(rows, plain)
+    assert runner.graph_replays >= 10 and runner.mixed_graph_replays > 0, (runner.graph_replays, runner.mixed_graph_replays)
+    assert worst <= LIMIT[dtype] and rms <= RMS_LIMIT[dtype], (worst, rms)
+
+
 @pytest.mark.parametrize("page_size", [4, 64])
 def test_other_page_sizes(models, page_size):
     raw, weights, requests, plain = models["A"]
