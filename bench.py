@@ -5,6 +5,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
                     [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 32768]
                     [--mixed-portions 16,64,248] [--other-shapes 7b,14b]
+    python bench.py --design polosun [--design-shapes 3b,7b] [--design-layers 12]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -27,6 +28,15 @@ holds decode at batch 1 and 64, at the main batch behind ``--long-contexts``
 tokens, and, for the ``--other-shapes`` of the family, decode at the main batch
 and context and the prefill, each with its share of the roofline in
 ``points_frac`` (the bytes and flops of its own shape).  ONE JSON line is printed.
+
+``--design polosun`` measures something else and leaves the above as it is: the
+Polosun design (layers of retention, latent attention and gated linear
+recurrence in turn, each with a dense feed-forward) beside the Qwen2.5 decoder
+of equal width, feed-forward size, vocabulary and layer count, both with
+``--design-layers`` layers and random weights: prefill of ``--prefill-tokens``
+tokens and decode at batch 1, ``--batch`` and 64 behind ``--context`` tokens,
+each with its share of the roofline of its own bytes and flops.  It prints one
+JSON line of its own.
 """
 
 from __future__ import annotations
@@ -218,6 +228,107 @@ def time_prefill(engine, config, tokens: int, seed: int) -> list[float]:
     return seconds
 
 
+def polosun_raw(shape: dict, layers: int) -> dict:
+    """A Polosun configuration with the width, feed-forward size and vocabulary of a Qwen2.5 shape and layers of
+    realistic proportions: retention heads of 128 x 256, latent attention with heads of 128 + 32 whose cache entry
+    (a latent of 96 and a turned part of 32) fills one 128-wide head of the attention kernels, a gated recurrence as
+    wide as the model in blocks of 256 channels with four taps."""
+    width = shape["hidden_size"]
+    mlp = {"kind": "dense", "ff": shape["intermediate_size"]}
+    kinds = [
+        {"type": "retention", "mlp": mlp,
+         "mixer": {"heads": width // 256, "dim": 128, "vdim": 256, "rot": {"base": 10000.0, "dims": 128},
+                   "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(width // 256 - 1, 1)) for h in range(width // 256)]}},
+        {"type": "latent_attention", "mlp": mlp,
+         "mixer": {"heads": width // 128, "dim": 128, "rot_dim": 32, "vdim": 128, "kv_rank": 96, "scale": 160 ** -0.5,
+                   "rot": {"base": 1000000.0, "dims": 32,
+                           "scaling": {"factor": 8.0, "fast": 32.0, "original": 4096, "slow": 1.0}}}},
+        {"type": "rglru", "mlp": mlp, "mixer": {"width": width, "blocks": width // 256, "conv": 4}},
+    ]
+    return {"architecture": "Polosun", "vocab": shape["vocab_size"], "width": width, "residual_mult": 0.5,
+            "norm": {"eps": 1e-6}, "layers": [kinds[i % 3] for i in range(layers)]}
+
+
+def polosun_costs(config, batch: int, context: float, tokens: int, elem: int) -> tuple[float, float]:
+    """(bytes one decode step has to move, flops of a prefill of ``tokens`` tokens) for a Polosun configuration:
+    every weight once (the embedding is only looked up), each request's latent cache read in both of its layouts,
+    each retention memory and recurrence state read and written in float32; products at two flops per weight and
+    token, attention over the latent entries, the memories' updates and read-outs."""
+    from cie_amd.parts.model import expected_tensors
+
+    expected = expected_tensors(config.model_spec())
+    weights = sum(int(__import__("math").prod(spec.shape)) for name, spec in expected.items() if name != "embed")
+    head = config.vocab_size * config.hidden_size
+    moved, attention = float(weights * elem), 0.0
+    for layer in config.raw["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "latent_attention":
+            entry = next(size for size in (32, 64, 96, 128, 256) if size >= m["kv_rank"] + m["rot_dim"])
+            moved += batch * context * 2 * entry * elem
+            attention += 2 * 2 * (tokens * (tokens + 1) / 2) * entry * m["heads"]
+        elif layer["type"] == "retention":
+            moved += batch * 2 * m["heads"] * m["dim"] * m["vdim"] * 4
+            attention += 2 * 2 * tokens * m["heads"] * m["dim"] * m["vdim"]
+        else:
+            moved += batch * 2 * m["width"] * m["conv"] * 4
+    return moved, 2.0 * tokens * (weights - head) + 2.0 * head + attention
+
+
+def compare_designs(args) -> int:
+    """``--design polosun``: see the module's text."""
+    import torch
+
+    from cie_amd.config import PolosunConfig, Qwen2Config
+    from cie_amd.workloads import SHAPES
+
+    elem = 2 if args.dtype == "bf16" else 4
+    steps, warmup, layers = args.steps, max(args.warmup, 1), args.design_layers
+    out = {}
+    for name in [n for n in args.design_shapes.split(",") if n]:
+        shape = SHAPES[name]
+        designs = {
+            "polosun": PolosunConfig.from_hf_config(polosun_raw(shape, layers)),
+            "qwen2": Qwen2Config.from_hf_config(dict(shape, num_hidden_layers=layers)),
+        }
+        out[name] = {}
+        for design, config in designs.items():
+            def costs(batch, context):
+                if design == "polosun":
+                    return polosun_costs(config, batch, context, args.prefill_tokens, elem)
+                return (decode_bytes(config, layers, batch, context, elem), prefill_flops(config, layers, args.prefill_tokens))
+
+            record = {}
+            print(f"[bench] {design} at the {name} widths, {layers} layers: prefill of {args.prefill_tokens}", file=sys.stderr, flush=True)
+            engine = make_engine(config, args.dtype, 1, args.prefill_tokens + 1, args.prefill_tokens)
+            seconds = statistics.median(time_prefill(engine, config, args.prefill_tokens, seed=99))
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+            record["prefill"] = {"tokens_per_s": round(args.prefill_tokens / seconds, 1), "ms": round(seconds * 1e3, 3),
+                                 "frac": round(costs(1, 1)[1] / seconds / PEAK_FLOPS[args.dtype], 4)}
+            for batch in sorted({1, args.batch, 64}):
+                print(f"[bench] {design} at the {name} widths: decode, batch {batch}, context {args.context}", file=sys.stderr, flush=True)
+                engine = make_engine(config, args.dtype, batch, args.context, args.prefill_tokens)
+                measured = decode_windows(engine, config, batch, args.context, steps, warmup, seed=batch)
+                del engine
+                gc.collect()
+                torch.cuda.empty_cache()
+                taken, mean_context = sorted(measured)[len(measured) // 2]
+                record[f"decode_b{batch}"] = {
+                    "tokens_per_s": round(batch * steps / taken, 2), "ms_per_step": round(taken / steps * 1e3, 4),
+                    "frac": round(costs(batch, mean_context)[0] / (taken / steps) / 1e9 / HBM_GBPS, 4)}
+            out[name][design] = record
+    print(json.dumps({
+        "metric": f"Polosun beside the Qwen2.5 decoder of equal width, feed-forward, vocabulary and {layers} layers",
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
+        "data": "synthetic (seeded uniform-random token ids, random weights N(0, 0.02))",
+        "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens, "page_size": PAGE,
+                   "polosun_layers": "retention, latent_attention, rglru in turn, each with a dense feed-forward"},
+        "shapes": out,
+    }))
+    return 0
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
@@ -239,10 +350,17 @@ def main(argv=None) -> int:
                              "(default 16,64,248; '' for none, as with --no-points)")
     parser.add_argument("--other-shapes", default="7b,14b",
                         help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
+    parser.add_argument("--design", default=None, choices=["polosun"],
+                        help="instead of the default record: this design beside the Qwen2.5 decoder of equal size")
+    parser.add_argument("--design-shapes", default="3b,7b", help="the Qwen2.5 shapes whose sizes the comparison takes")
+    parser.add_argument("--design-layers", type=int, default=12, help="layers of both models in the comparison")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not run (this engine is single-GPU)")
         return 2
+
+    if args.design is not None:
+        return compare_designs(args)
 
     import torch
 

@@ -10,7 +10,8 @@
 // It serves per-head products (a query folded into a shared latent space and back out of it) and gates made from
 // a channel's own block.  Operands are float32 or bfloat16, sums are float32 fused multiply-adds in one fixed order
 // of k (blocks of 256 summed, then the blocks' sums), so a row's result does not depend on the other rows; the
-// result is float32 or the operands' type.  64 x 64 results per workgroup, slices of 16 k through LDS.
+// result is float32 or the operands' type.  64 x 64 results per workgroup, slices of 16 k through LDS; up to 16 rows
+// take a form of their own (below) whose sums have another fixed order, again the same for every row.
 #include "common.h"
 
 namespace {
@@ -88,6 +89,65 @@ block_linear_kernel(const TA* __restrict__ A, long lda, long a_block, const TA* 
         }
     }
 }
+// Up to 16 rows (a decode step): the weights are the traffic.  One wave per result column at a time (each wave takes
+// kRowsOutputs / 4 columns in turn): its lanes stride over k, so a weight row is read in whole segments, the few rows of
+// A come through the cache, and the lanes' shares meet in a wave-wide sum; lane m stores row m's result.
+constexpr int kRowsOutputs = 16;
+
+template <typename TA, typename TC, int MR>
+__global__ void __launch_bounds__(256)
+block_linear_rows_kernel(const TA* __restrict__ A, long lda, long a_block, const TA* __restrict__ W,
+                         const TA* __restrict__ bias, TC* __restrict__ C, long ldc, long c_block,
+                         const TA* __restrict__ gate, long ldg, long g_block, int M, int N, int K) {
+    const int b = blockIdx.y;
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const TA* a_base = A + static_cast<size_t>(b) * a_block;
+    for (int turn = 0; turn < kRowsOutputs / 4; ++turn) {
+        const int n = blockIdx.x * kRowsOutputs + turn * 4 + wave;
+        if (n >= N) return;  // (a wave leaves whole)
+        const TA* w_row = W + (static_cast<size_t>(b) * N + n) * K;
+        float acc[MR];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+        for (int k = lane; k < K; k += kWave) {
+            const float w = to_float(w_row[k]);
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (m < M) acc[m] = fmaf(to_float(a_base[static_cast<size_t>(m) * lda + k]), w, acc[m]);
+        }
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const float total = wave_sum(acc[m]);
+            if (lane == m && m < M) {
+                float v = total;
+                if (bias) v += to_float(bias[static_cast<size_t>(b) * N + n]);
+                if (gate) {
+                    const float g = to_float(gate[static_cast<size_t>(m) * ldg + static_cast<size_t>(b) * g_block + n]);
+                    v *= 1.0f / (1.0f + expf(-g));
+                }
+                C[static_cast<size_t>(m) * ldc + static_cast<size_t>(b) * c_block + n] = from_float<TC>(v);
+            }
+        }
+    }
+}
+
+template <typename TA, typename TC>
+int launch_rows(hipStream_t s, const void* A, long lda, long a_block, const void* W, const void* bias, void* C, long ldc,
+                long c_block, const void* gate, long ldg, long g_block, int M, int N, int K, int B) {
+    dim3 grid((N + kRowsOutputs - 1) / kRowsOutputs, B);
+#define CIE_ROWS(MR)                                                                                                   \
+    block_linear_rows_kernel<TA, TC, MR><<<grid, 256, 0, s>>>(                                                         \
+        static_cast<const TA*>(A), lda, a_block, static_cast<const TA*>(W), static_cast<const TA*>(bias),              \
+        static_cast<TC*>(C), ldc, c_block, static_cast<const TA*>(gate), ldg, g_block, M, N, K)
+    if (M <= 1) CIE_ROWS(1);
+    else if (M <= 2) CIE_ROWS(2);
+    else if (M <= 4) CIE_ROWS(4);
+    else if (M <= 8) CIE_ROWS(8);
+    else CIE_ROWS(16);
+#undef CIE_ROWS
+    return cie_after_launch();
+}
 }  // namespace
 
 // dtype: type of A, W, bias and gate; out_f32: the result is float32 whatever the operands' type
@@ -100,6 +160,12 @@ CIE_API int cie_block_linear(void* stream, int dtype, int out_f32, const void* A
     if (grid_y > 65535) return CIE_BAD_ARGUMENT;
     dim3 grid((N + TN - 1) / TN, grid_y, B);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (M <= 16) {
+        if (dtype == CIE_F32) return launch_rows<float, float>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
+        if (dtype == CIE_BF16 && out_f32) return launch_rows<bf16_t, float>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
+        if (dtype == CIE_BF16) return launch_rows<bf16_t, bf16_t>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
+        return CIE_BAD_ARGUMENT;
+    }
     if (dtype == CIE_F32)
         block_linear_kernel<float, float><<<grid, 256, 0, s>>>(
             static_cast<const float*>(A), lda, a_block, static_cast<const float*>(W), static_cast<const float*>(bias),

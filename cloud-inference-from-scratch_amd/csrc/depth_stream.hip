@@ -31,11 +31,16 @@ __global__ void depth_stream_kernel(const float* __restrict__ x, const T* __rest
         }
         if (newest >= 0) history[static_cast<size_t>(newest) * layer_stride + row + h] = v;
         if (terms > 0) {
+            // (the loads of the earlier layers' rows do not depend on one another: none stands behind a condition,
+            // so that they travel together; the row just made comes from its register, last)
             float acc = 0.f;
-            for (int j = 0; j < terms; ++j) {
-                const float past = j == newest ? v : history[static_cast<size_t>(j) * layer_stride + row + h];
-                acc = fmaf(weights[j], past, acc);
-            }
+            const float* past = history + row + h;
+            const int own = (newest >= 0 && newest < terms) ? newest : terms;
+#pragma unroll 4
+            for (int j = 0; j < own; ++j) acc = fmaf(weights[j], past[static_cast<size_t>(j) * layer_stride], acc);
+#pragma unroll 4
+            for (int j = own + 1; j < terms; ++j) acc = fmaf(weights[j], past[static_cast<size_t>(j) * layer_stride], acc);
+            if (own < terms) acc = fmaf(weights[own], v, acc);
             v = acc;
         }
         if (stream) stream[row + h] = v;
@@ -62,7 +67,10 @@ CIE_API int cie_depth_stream(void* stream_handle, int dtype, const float* x, con
     if (branch_b && !branch_a) return CIE_BAD_ARGUMENT;
     if (rows == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream_handle);
-    const int threads = hidden >= 1024 ? 256 : 128;
+    // few rows (a decode step): a row is one workgroup's, so its width is spread over as many threads as it has
+    // numbers, up to 1,024; many rows fill the GPU with smaller workgroups
+    int threads = hidden >= 1024 ? 256 : 128;
+    if (rows <= 128) threads = hidden >= 1024 ? 1024 : hidden >= 512 ? 512 : threads;
     if (dtype == CIE_F32)
         depth_stream_kernel<float><<<rows, threads, hidden * sizeof(float), s>>>(
             x, static_cast<const float*>(branch_a), static_cast<const float*>(branch_b), mult, history, layer_stride,

@@ -922,24 +922,27 @@ def latent_rows(proj: torch.Tensor, weight: torch.Tensor, heads: int, plain: int
 
 
 RETENTION_ROWS = (4, 8, 16, 32)  # rows of a head's memory that one thread keeps in registers
+RETENTION_SLICE = 64             # value columns of a head that one workgroup takes
 RETENTION_LDS_FLOATS = 15 * 1024
 
 
-def plan_retention(dim: int, vdim: int) -> tuple[int, int, int]:
-    """(rows per thread, groups of threads, tokens per chunk) of the retention kernel for heads of ``dim`` x ``vdim``."""
-    if vdim > 1024:
-        raise ValueError(f"value heads of up to 1024 numbers, not {vdim}")
-    most_groups = max(1, min(dim, 1024 // vdim))
-    need = -(-dim // most_groups)
-    rows = next((r for r in RETENTION_ROWS if r >= need), None)
+def plan_retention(dim: int, vdim: int) -> tuple[int, int, int, int]:
+    """(rows per thread, groups of threads, value columns per workgroup, tokens per chunk) of the retention kernel
+    for heads of ``dim`` x ``vdim``: workgroups of up to 512 threads where the rows allow it (1,024 otherwise)."""
+    if dim < 1 or vdim < 1:
+        raise ValueError("head sizes must be positive")
+    piece = min(vdim, RETENTION_SLICE)
+    rows = next((r for r in RETENTION_ROWS if -(-dim // r) * piece <= 512), None)
+    if rows is None:
+        rows = next((r for r in RETENTION_ROWS if -(-dim // r) * piece <= 1024), None)
     if rows is None:
         raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's registers")
     groups = -(-dim // rows)
-    per_token = 2 * dim + vdim + groups * vdim
+    per_token = 2 * groups * rows + piece + groups * piece
     chunk = min(32, RETENTION_LDS_FLOATS // per_token)
     if chunk < 1:
         raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's LDS")
-    return rows, groups, chunk
+    return rows, groups, piece, chunk
 
 
 def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optional[torch.Tensor],
@@ -970,14 +973,15 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
         _gpu(name, meta, torch.int32, 1)
         if meta.shape[0] < least:
             raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
-    rows, groups, chunk = plan_retention(dim, vdim)
+    rows, groups, piece, chunk = plan_retention(dim, vdim)
+    raw = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
     ldp = proj.stride(0) if tokens > 1 else max(proj.stride(0), proj.shape[1])
     _run("cie_retention", load_library().cie_retention(
         _stream(), _i(_code(proj.dtype)), _ptr(proj), ldp, _i(q_off), _i(k_off), _i(v_off), _i(g_off),
         _ptr(cos if rot else None), _ptr(sin if rot else None), _i(rot), _ptr(decay), _ptr(state), _ptr(seq_slot),
-        _ptr(seq_start), _ptr(q_start_loc), _ptr(out), _i(sequences), _i(heads), _i(dim), _i(vdim), _i(rows), _i(groups),
-        _i(chunk), _f(eps), _f(key_scale)))
+        _ptr(seq_start), _ptr(q_start_loc), _ptr(raw), _ptr(out), _i(tokens), _i(sequences), _i(heads), _i(dim), _i(vdim),
+        _i(rows), _i(groups), _i(piece), _i(chunk), _f(eps), _f(key_scale)))
     return out
 
 
@@ -1017,11 +1021,13 @@ def causal_conv(x: torch.Tensor, taps_w: torch.Tensor, bias: Optional[torch.Tens
 
 def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, block_width: int,
                      rate: torch.Tensor, state: torch.Tensor, past: torch.Tensor, seq_slot: torch.Tensor,
-                     q_start_loc: torch.Tensor, sequences: int, taps: int) -> torch.Tensor:
+                     q_start_loc: torch.Tensor, sequences: int, taps: int, segments: int = 1) -> torch.Tensor:
     """The gated linear recurrence of ``csrc/recurrent.hip`` over a step's tokens: per channel
     ``a = exp(rate * sigmoid(r))``, ``S = a * S + sqrt(1 - a^2) * sigmoid(i) * u``, ``out = S * gelu_tanh(y_pre)``,
     with r and i from ``gates`` (float32 [T, 2C], per block of ``block_width`` channels its r then its i).  ``state``
-    float32 [slots, C]; ``past`` float32 [slots, max(taps - 1, 1), C] is moved on with the step's ``x_in``."""
+    float32 [slots, C]; ``past`` float32 [slots, max(taps - 1, 1), C] is moved on with the step's ``x_in``.
+    ``segments`` (1 to 16) stretches of a sequence's tokens run side by side and are joined by the recurrence's
+    own linearity (for long portions; the result differs from the walk in order by float32 rounding only)."""
     tokens, channels = u.shape
     for name, t in (("y_pre", y_pre), ("x_in", x_in)):
         if not (t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.dtype == u.dtype and tuple(t.shape) == (tokens, channels)):
@@ -1033,7 +1039,7 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
     _gpu("past", past, torch.float32, 3)
     if (tuple(gates.shape) != (tokens, 2 * channels) or rate.shape[0] != channels or state.shape[1] != channels
             or tuple(past.shape[1:]) != (max(taps - 1, 1), channels) or channels % block_width
-            or not 1 <= taps <= MAX_CONV_TAPS):
+            or not 1 <= taps <= MAX_CONV_TAPS or not 1 <= segments <= 16):
         raise ValueError("gates, rate, state or past do not fit the channels")
     for name, meta, least in (("seq_slot", seq_slot, sequences), ("q_start_loc", q_start_loc, sequences + 1)):
         _gpu(name, meta, torch.int32, 1)
@@ -1044,5 +1050,5 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
     _run("cie_gated_recurrence", load_library().cie_gated_recurrence(
         _stream(), _i(_code(u.dtype)), _ptr(y_pre), ld(y_pre), _ptr(x_in), ld(x_in), _ptr(u), _ptr(gates),
         _i(block_width), _ptr(rate), _ptr(state), _ptr(past), _ptr(seq_slot), _ptr(q_start_loc), _ptr(out),
-        _i(sequences), _i(channels), _i(taps)))
+        _i(sequences), _i(channels), _i(taps), _i(segments)))
     return out

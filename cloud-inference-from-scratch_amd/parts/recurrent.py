@@ -87,6 +87,9 @@ class Retention(Part):
         return linear(out, self.w_o)
 
 
+SCAN_SEGMENT_TOKENS = 64  # portions from which the recurrence's tokens are cut into stretches
+
+
 class GatedLinearRecurrence(Part):
     graph_safe = True
 
@@ -137,8 +140,10 @@ class GatedLinearRecurrence(Part):
         y_pre, x_in = proj[:, :w], proj[:, w:]
         u = ops.causal_conv(x_in, self.conv_w, self.conv_b, past, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
         gates = ops.block_linear(u, self.w_gates, self.b_gates, out_dtype=torch.float32)
+        # long portions run as stretches side by side (the portion lengths are the host's, and a captured step's own)
+        segments = 16 if batch.max_q_len >= SCAN_SEGMENT_TOKENS else 1
         out = ops.gated_recurrence(y_pre, x_in, u, gates, w // self.blocks, self.rate, state, past, batch.seq_slot,
-                                   batch.q_start_loc, batch.sequences, self.taps)
+                                   batch.q_start_loc, batch.sequences, self.taps, segments)
         return linear(out, self.w_o)
 
 

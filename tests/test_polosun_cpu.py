@@ -194,9 +194,9 @@ def test_plain_model_composes_branches_and_depth_average():
 def test_retention_kernel_plan_fits_its_limits():
     from cie_amd.kernels import ops
 
-    for dim, vdim in ((32, 64), (8, 40), (128, 256), (256, 64), (4, 72), (32, 1024)):
-        rows, groups, chunk = ops.plan_retention(dim, vdim)
-        assert rows in ops.RETENTION_ROWS and rows * groups >= dim and vdim * groups <= 1024 + 63
-        assert chunk >= 1 and chunk * (2 * dim + vdim + groups * vdim) <= ops.RETENTION_LDS_FLOATS
+    for dim, vdim in ((32, 64), (8, 40), (128, 256), (256, 64), (4, 72), (32, 1024), (512, 512), (3, 5)):
+        rows, groups, piece, chunk = ops.plan_retention(dim, vdim)
+        assert rows in ops.RETENTION_ROWS and rows * groups >= dim and piece * groups <= 1024 and piece <= min(vdim, 64)
+        assert chunk >= 1 and chunk * (2 * rows * groups + piece + groups * piece) <= ops.RETENTION_LDS_FLOATS
     with pytest.raises(ValueError):
-        ops.plan_retention(256, 512)
+        ops.plan_retention(1024, 64)
