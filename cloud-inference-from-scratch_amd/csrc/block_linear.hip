@@ -89,10 +89,11 @@ block_linear_kernel(const TA* __restrict__ A, long lda, long a_block, const TA* 
         }
     }
 }
-// Up to 16 rows (a decode step): the weights are the traffic.  One wave per result column at a time (each wave takes
-// kRowsOutputs / 4 columns in turn): its lanes stride over k, so a weight row is read in whole segments, the few rows of
-// A come through the cache, and the lanes' shares meet in a wave-wide sum; lane m stores row m's result.
-constexpr int kRowsOutputs = 16;
+// Up to 16 rows (a decode step): the weights are the traffic.  One wave per result column (a column's work is a chain
+// of a few dependent loads and a sum across lanes, so what counts is how many columns are under way at once): its lanes
+// stride over k, so a weight row is read in whole segments, the few rows of A come through the cache, and the lanes'
+// shares meet in a wave-wide sum; lane m stores row m's result.
+constexpr int kRowsOutputs = 4;
 
 template <typename TA, typename TC, int MR>
 __global__ void __launch_bounds__(256)

@@ -5,7 +5,7 @@
 // 1. retention: a memory S [dim, vdim] per head that fades by a fixed factor per token,
 //        S_t = decay * S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t,
 //    q and k turned by the token's position (the first `rot` dimensions of a head, pair (i, i + rot/2)), k scaled
-//    after the turn; o_t divided by its root mean square over the head and multiplied by silu(gate) (a second kernel).
+//    after the turn; o_t divided by its root mean square over the head and multiplied by silu(gate).
 // 2. a causal convolution over each channel's own last `taps` inputs, the inputs of the tokens before the step taken
 //    from the state.
 // 3. a gated linear recurrence per channel,
@@ -25,98 +25,173 @@ __device__ __forceinline__ float gelu_tanh(float z) {
 }
 
 // ---------------------------------------------------------------------------------------------- retention
-// A column of the memory never meets another column, so one workgroup takes (sequence, head, slice of up to 64
-// value columns).  Thread (column v, group g) keeps rows g * DS .. g * DS + DS - 1 of column v in registers.
-// Tokens go in chunks: the chunk's turned queries and keys (rows padded with zeros to groups * DS numbers, so that
-// a thread reads its DS numbers as 16-byte pieces without a condition) and its values are staged in LDS as float32,
-// every thread walks the chunk's tokens in order (no barrier between tokens), and the groups' shares of o_t are
-// summed into a float32 buffer [tokens, heads * vdim].  The head's norm and the gate are a second, small kernel:
-// they need all slices of a head.
+// Three kernels.  (a) Every token's queries and keys, turned by its position, the keys scaled, as float32 rows padded
+// with zeros to `padded` numbers per head: [tokens, heads, 2, padded].  (b) The walk over the tokens, below.  (c) The
+// head's norm and the gate, which need all value columns of a head.
+//
+// (b) A column of the memory never meets another column, and o_t is a sum over the memory's rows, so one workgroup
+// takes (sequence, head, slice of up to 64 value columns, part of the rows) and the parts' shares of o_t are added
+// up by (c): as many parts as give every compute unit a workgroup (a prompt of one sequence with 8 heads of 128 x 256
+// would otherwise keep 32 of 256 units busy, each walking its 2,048 tokens at 64 multiply-adds per thread and token).
+// Thread (column v, group g) keeps rows r0 + g * DS .. + DS - 1 of column v in registers.  Tokens go in chunks:
+// the chunk's queries, keys and values are staged in LDS, every thread walks the chunk's tokens in order (no
+// barrier between tokens; a thread reads its DS numbers of a query as 16-byte pieces), and the groups' shares are
+// summed into the part's float32 plane [tokens, heads * vdim].  The next chunk's numbers are fetched into
+// registers before the walk over the current one starts, so that their way from memory is hidden behind it.
+template <typename T>
+__global__ void __launch_bounds__(256)
+retention_turn_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off, const float* __restrict__ cos_table,
+                      const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
+                      float* __restrict__ turned, int heads, int dim, int padded, float key_scale) {
+    const int token = blockIdx.x;
+    const int half = rot / 2;
+    const T* row = proj + static_cast<size_t>(token) * ldp;
+    const size_t at = static_cast<size_t>(positions[token]) * half;
+    for (int idx = threadIdx.x; idx < heads * padded; idx += blockDim.x) {
+        const int head = idx / padded;
+        const int d = idx - head * padded;
+        float qv = 0.f, kv = 0.f;
+        if (d < dim) {
+            const T* qh = row + q_off + head * dim;
+            const T* kh = row + k_off + head * dim;
+            qv = to_float(qh[d]);
+            kv = to_float(kh[d]);
+            if (d < rot) {
+                const int i = d < half ? d : d - half;
+                const float c = cos_table[at + i], s = sin_table[at + i];
+                if (d < half) {
+                    qv = qv * c - to_float(qh[d + half]) * s;
+                    kv = kv * c - to_float(kh[d + half]) * s;
+                } else {
+                    qv = qv * c + to_float(qh[i]) * s;
+                    kv = kv * c + to_float(kh[i]) * s;
+                }
+            }
+        }
+        float* dst = turned + ((static_cast<size_t>(token) * heads + head) * 2) * padded + d;
+        dst[0] = qv;
+        dst[padded] = kv * key_scale;
+    }
+}
+
+typedef float piece_t __attribute__((ext_vector_type(4)));  // 16 bytes that stay in registers (as a struct of four
+                                                            // floats, the pieces fetched ahead went through scratch memory)
+
+constexpr int kFetchPieces = 6;  // 16-byte pieces of a chunk's queries and keys that a thread fetches ahead
+constexpr int kFetchValues = 12; // ... and values
+
+// the chunk that starts at token `from`: this thread's pieces into its registers.  Every load stands in straight-line
+// code without a condition (a piece or value past the chunk's end reads the chunk's last one again, a column past the
+// head's last its last): behind a load under a condition the compiler waits for it before it issues the next, and
+// the eighteen loads of a thread became eighteen round trips to memory per chunk.
+#define CIE_RETENTION_FETCH(from)                                                                                     \
+    {                                                                                                                 \
+        const int fetch_n = min(chunk, count - (from));                                                               \
+        _Pragma("unroll") for (int i = 0; i < kFetchPieces; ++i) {                                                    \
+            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * pieces - 1);                \
+            const int t = idx / pieces;                                                                               \
+            const int piece = idx - t * pieces;                                                                       \
+            const int side = piece / (rows / 4); /* 0: the query, 1: the key */                                       \
+            ahead[i] = *reinterpret_cast<const piece_t*>(                                                             \
+                turned + ((static_cast<size_t>(first + (from) + t) * heads + head) * 2 + side) * padded + r0 +        \
+                (piece - side * (rows / 4)) * 4);                                                                     \
+        }                                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < kFetchValues; ++i) {                                                    \
+            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * slice - 1);                 \
+            const int t = idx / slice;                                                                                \
+            const int c = min(v0 + idx - t * slice, vdim - 1);                                                        \
+            ahead_v[i] = to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]);     \
+        }                                                                                                             \
+    }
+
 template <typename T, int DS>
-__global__ void __launch_bounds__(1024)
-retention_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off, int v_off,
-                 const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot,
+__global__ void __launch_bounds__(512)
+retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* __restrict__ turned,
                  const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seq_slot,
-                 const int* __restrict__ seq_start, const int* __restrict__ q_start_loc, float* __restrict__ raw,
-                 int heads, int dim, int vdim, int slice, int groups, int chunk, float key_scale) {
+                 const int* __restrict__ q_start_loc, float* __restrict__ raw, long plane,
+                 int heads, int dim, int vdim, int slice, int slices, int groups, int padded, int chunk) {
     extern __shared__ float4 lds4[];
     float* lds = reinterpret_cast<float*>(lds4);
-    const int padded = groups * DS;
-    float* q_s = lds;                          // [chunk][padded]
-    float* k_s = q_s + chunk * padded;         // [chunk][padded]
-    float* v_s = k_s + chunk * padded;         // [chunk][slice]
+    const int rows = groups * DS;              // rows of the memory that this workgroup keeps
+    float* qk_s = lds;                         // [chunk][2][rows]: a token's query, then its key
+    float* v_s = qk_s + chunk * 2 * rows;      // [chunk][slice]
     float* o_s = v_s + chunk * slice;          // [groups][chunk][slice]
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
-    const int v0 = blockIdx.z * slice;
+    const int part = blockIdx.z / slices;
+    const int v0 = (blockIdx.z - part * slices) * slice;
+    const int r0 = part * rows;
     const int first = q_start_loc[seq];
     const int count = q_start_loc[seq + 1] - first;
-    const int start = seq_start[seq];
     const int slot = seq_slot[seq];
     const int col = threadIdx.x % slice;
     const int grp = threadIdx.x / slice;
     const bool owner = grp < groups && v0 + col < vdim;
-    const int d0 = grp * DS;
+    const int d0 = r0 + grp * DS;
     const float fade = decay[head];
-    const int half = rot / 2;
+    const int pieces = 2 * rows / 4;           // 16-byte pieces of one token's query and key rows
     float* mem = state + ((static_cast<size_t>(slot) * heads + head) * dim) * vdim + v0 + col;
+    float* mine = raw + static_cast<size_t>(part) * plane;
     float S[DS];
 #pragma unroll
     for (int r = 0; r < DS; ++r) S[r] = (owner && d0 + r < dim) ? mem[static_cast<size_t>(d0 + r) * vdim] : 0.f;
+    piece_t ahead[kFetchPieces];
+    float ahead_v[kFetchValues];
+    if (count > 0) CIE_RETENTION_FETCH(0)
     for (int c0 = 0; c0 < count; c0 += chunk) {
         const int cn = min(chunk, count - c0);
-        for (int idx = threadIdx.x; idx < cn * padded; idx += blockDim.x) {
-            const int t = idx / padded;
-            const int d = idx - t * padded;
-            float qv = 0.f, kv = 0.f;
-            if (d < dim) {
-                const T* row = proj + static_cast<size_t>(first + c0 + t) * ldp;
-                const T* qh = row + q_off + head * dim;
-                const T* kh = row + k_off + head * dim;
-                qv = to_float(qh[d]);
-                kv = to_float(kh[d]);
-                if (d < rot) {
-                    const int i = d < half ? d : d - half;
-                    const size_t at = static_cast<size_t>(start + c0 + t) * half + i;
-                    const float c = cos_table[at], s = sin_table[at];
-                    if (d < half) {
-                        qv = qv * c - to_float(qh[d + half]) * s;
-                        kv = kv * c - to_float(kh[d + half]) * s;
-                    } else {
-                        qv = qv * c + to_float(qh[i]) * s;
-                        kv = kv * c + to_float(kh[i]) * s;
-                    }
-                }
-            }
-            q_s[idx] = qv;
-            k_s[idx] = kv * key_scale;
+#pragma unroll
+        for (int i = 0; i < kFetchPieces; ++i) {
+            const int idx = threadIdx.x + i * blockDim.x;
+            if (idx < cn * pieces) reinterpret_cast<piece_t*>(qk_s)[idx] = ahead[i];
         }
-        for (int idx = threadIdx.x; idx < cn * slice; idx += blockDim.x) {
-            const int t = idx / slice;
-            const int c = idx - t * slice;
-            v_s[idx] = v0 + c < vdim
-                           ? to_float(proj[static_cast<size_t>(first + c0 + t) * ldp + v_off + head * vdim + v0 + c]) : 0.f;
+#pragma unroll
+        for (int i = 0; i < kFetchValues; ++i) {
+            const int idx = threadIdx.x + i * blockDim.x;
+            if (idx < cn * slice) v_s[idx] = ahead_v[i];
         }
         __syncthreads();
+        if (c0 + chunk < count) CIE_RETENTION_FETCH(c0 + chunk)
         if (owner) {
+            // (a token's numbers are read from LDS while the token before it is worked on: with one wave per SIMD
+            // nothing else would hide the way from LDS, and it is as long as the arithmetic of a token)
+            const float* q_base = qk_s + grp * DS;
+            float4 q_next[DS / 4], k_next[DS / 4];
+            float v_next = v_s[col];
+#pragma unroll
+            for (int r = 0; r < DS / 4; ++r) {
+                q_next[r] = reinterpret_cast<const float4*>(q_base)[r];
+                k_next[r] = reinterpret_cast<const float4*>(q_base + rows)[r];
+            }
             for (int t = 0; t < cn; ++t) {
-                const float vt = v_s[t * slice + col];
-                const float4* qt = reinterpret_cast<const float4*>(q_s + t * padded + d0);
-                const float4* kt = reinterpret_cast<const float4*>(k_s + t * padded + d0);
-                float acc = 0.f;
+                float4 q_now[DS / 4], k_now[DS / 4];
+                const float vt = v_next;
 #pragma unroll
                 for (int r = 0; r < DS / 4; ++r) {
-                    const float4 k4 = kt[r], q4 = qt[r];
+                    q_now[r] = q_next[r];
+                    k_now[r] = k_next[r];
+                }
+                const int ahead_t = min(t + 1, cn - 1);  // (the last token is read twice: no condition around the reads)
+                v_next = v_s[ahead_t * slice + col];
+#pragma unroll
+                for (int r = 0; r < DS / 4; ++r) {
+                    q_next[r] = reinterpret_cast<const float4*>(q_base + ahead_t * 2 * rows)[r];
+                    k_next[r] = reinterpret_cast<const float4*>(q_base + ahead_t * 2 * rows + rows)[r];
+                }
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+                for (int r = 0; r < DS / 4; ++r) {
+                    const float4 k4 = k_now[r], q4 = q_now[r];
                     S[4 * r + 0] = fmaf(fade, S[4 * r + 0], k4.x * vt);
                     S[4 * r + 1] = fmaf(fade, S[4 * r + 1], k4.y * vt);
                     S[4 * r + 2] = fmaf(fade, S[4 * r + 2], k4.z * vt);
                     S[4 * r + 3] = fmaf(fade, S[4 * r + 3], k4.w * vt);
-                    acc = fmaf(S[4 * r + 0], q4.x, acc);
-                    acc = fmaf(S[4 * r + 1], q4.y, acc);
-                    acc = fmaf(S[4 * r + 2], q4.z, acc);
-                    acc = fmaf(S[4 * r + 3], q4.w, acc);
+                    a0 = fmaf(S[4 * r + 0], q4.x, a0);
+                    a1 = fmaf(S[4 * r + 1], q4.y, a1);
+                    a2 = fmaf(S[4 * r + 2], q4.z, a2);
+                    a3 = fmaf(S[4 * r + 3], q4.w, a3);
                 }
-                o_s[(grp * chunk + t) * slice + col] = acc;
+                o_s[(grp * chunk + t) * slice + col] = (a0 + a1) + (a2 + a3);
             }
         }
         __syncthreads();
@@ -126,7 +201,7 @@ retention_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off, int
             if (v0 + c >= vdim) continue;
             float o = 0.f;
             for (int g = 0; g < groups; ++g) o += o_s[(g * chunk + t) * slice + c];
-            raw[static_cast<size_t>(first + c0 + t) * heads * vdim + head * vdim + v0 + c] = o;
+            mine[static_cast<size_t>(first + c0 + t) * heads * vdim + head * vdim + v0 + c] = o;
         }
         __syncthreads();
     }
@@ -135,20 +210,26 @@ retention_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off, int
         for (int r = 0; r < DS; ++r)
             if (d0 + r < dim) mem[static_cast<size_t>(d0 + r) * vdim] = S[r];
 }
+#undef CIE_RETENTION_FETCH
 
 // o / sqrt(mean(o^2) over the head + eps) * silu(gate): one wave per (token, head)
 template <typename T>
 __global__ void __launch_bounds__(256)
-retention_norm_kernel(const float* __restrict__ raw, const T* __restrict__ proj, long ldp, int g_off,
+retention_norm_kernel(float* __restrict__ raw, long plane, int parts, const T* __restrict__ proj, long ldp, int g_off,
                       T* __restrict__ out, int tokens, int heads, int vdim, float eps) {
     const int item = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (item >= tokens * heads) return;  // (whole waves leave together)
     const int lane = threadIdx.x % kWave;
     const int token = item / heads;
     const int head = item - token * heads;
-    const float* o = raw + static_cast<size_t>(token) * heads * vdim + head * vdim;
+    float* o = raw + static_cast<size_t>(token) * heads * vdim + head * vdim;
     float sum_sq = 0.f;
-    for (int c = lane; c < vdim; c += kWave) sum_sq += o[c] * o[c];
+    for (int c = lane; c < vdim; c += kWave) {
+        float v = o[c];
+        for (int p = 1; p < parts; ++p) v += o[static_cast<size_t>(p) * plane + c];  // (the parts in their order)
+        o[c] = v;  // (this lane's own column: it reads it again below)
+        sum_sq += v * v;
+    }
     const float inv = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(vdim) + eps);
     const T* gate = proj + static_cast<size_t>(token) * ldp + g_off + head * vdim;
     T* dst = out + static_cast<size_t>(token) * heads * vdim + head * vdim;
@@ -159,13 +240,13 @@ retention_norm_kernel(const float* __restrict__ raw, const T* __restrict__ proj,
 }
 
 template <typename T, int DS>
-int launch_retention(hipStream_t s, dim3 grid, int threads, size_t lds, const void* proj, long ldp, int q_off, int k_off,
-                     int v_off, const float* cos_table, const float* sin_table, int rot, const float* decay,
-                     float* state, const int* seq_slot, const int* seq_start, const int* q_start_loc, float* raw, int heads,
-                     int dim, int vdim, int slice, int groups, int chunk, float key_scale) {
-    retention_kernel<T, DS><<<grid, threads, lds, s>>>(
-        static_cast<const T*>(proj), ldp, q_off, k_off, v_off, cos_table, sin_table, rot, decay, state, seq_slot,
-        seq_start, q_start_loc, raw, heads, dim, vdim, slice, groups, chunk, key_scale);
+int launch_retention(hipStream_t s, dim3 grid, int threads, size_t lds, const void* proj, long ldp, int v_off,
+                     const float* turned, const float* decay, float* state, const int* seq_slot, const int* q_start_loc,
+                     float* raw, long plane, int heads, int dim, int vdim, int slice, int slices, int groups, int padded,
+                     int chunk) {
+    retention_kernel<T, DS><<<grid, threads, lds, s>>>(static_cast<const T*>(proj), ldp, v_off, turned, decay, state,
+                                                      seq_slot, q_start_loc, raw, plane, heads, dim, vdim, slice, slices,
+                                                      groups, padded, chunk);
     return cie_after_launch();
 }
 
@@ -197,13 +278,14 @@ causal_conv_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ taps
 // S_t = a_t S_(t-1) + x_t is linear in S, so a sequence's tokens are cut into `segments` stretches that run side by
 // side: thread (channel, stretch) first folds its stretch into (A, B) with S_out = A S_in + B, the stretches before
 // it give its S_in (a chain of at most `segments` multiply-adds), and a second walk over the stretch makes the
-// outputs.  With one stretch this is the plain walk in order.  64 channels per workgroup.
+// outputs.  With one stretch this is the plain walk in order.  16 channels per workgroup when cut into stretches.
 constexpr int kMaxTaps = 16;
 constexpr int kMaxSegments = 16;
-constexpr int kScanChannels = 64;
 
-template <typename T>
-__global__ void __launch_bounds__(kScanChannels * kMaxSegments)
+// (kScanChannels channels a workgroup: 64 for the walk in order; 16 when cut into stretches, where the arithmetic per
+// token bounds the kernel and more workgroups mean more compute units at work)
+template <typename T, int kScanChannels>
+__global__ void __launch_bounds__(kScanChannels == 64 ? 64 : kScanChannels * kMaxSegments)
 gated_recurrence_kernel(const T* __restrict__ y_pre, long ldy, const T* __restrict__ x_in, long ldx,
                         const T* __restrict__ u, const float* __restrict__ gates, int block_width,
                         const float* __restrict__ rate, float* __restrict__ state, float* __restrict__ past,
@@ -238,7 +320,8 @@ gated_recurrence_kernel(const T* __restrict__ y_pre, long ldy, const T* __restri
     if (segments > 1) {
         float A = 1.f, B = 0.f;
         if (live)
-            for (int t = t0; t < t1; ++t) {
+#pragma unroll 4
+            for (int t = t0; t < t1; ++t) {  // (four tokens per turn: their loads travel together)
                 float a, x;
                 step(t, a, x);
                 B = fmaf(a, B, x);
@@ -250,6 +333,7 @@ gated_recurrence_kernel(const T* __restrict__ y_pre, long ldy, const T* __restri
         for (int before = 0; before < seg; ++before) S = fmaf(a_s[before][lane], S, b_s[before][lane]);
     }
     if (!live) return;
+#pragma unroll 4
     for (int t = t0; t < t1; ++t) {
         float a, x;
         step(t, a, x);
@@ -279,32 +363,46 @@ gated_recurrence_kernel(const T* __restrict__ y_pre, long ldy, const T* __restri
 
 CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, int q_off, int k_off, int v_off, int g_off,
                           const float* cos_table, const float* sin_table, int rot, const float* decay, float* state,
-                          const int* seq_slot, const int* seq_start, const int* q_start_loc, float* raw, void* out,
-                          int tokens, int sequences, int heads, int dim, int vdim, int rows_per_thread, int groups,
-                          int slice, int chunk, float eps, float key_scale) {
+                          const int* seq_slot, const int* positions, const int* q_start_loc, float* turned, float* raw,
+                          void* out, int tokens, int sequences, int heads, int dim, int vdim, int rows_per_thread,
+                          int groups, int parts, int slice, int chunk, float eps, float key_scale) {
     if (sequences < 0 || tokens < 0 || heads <= 0 || heads > 65535 || dim <= 0 || vdim <= 0 || groups <= 0 || chunk <= 0 ||
-        slice <= 0 || slice > vdim || rot < 0 || rot % 2 || rot > dim || (rot > 0 && (!cos_table || !sin_table)) ||
-        !(eps > 0.f) || static_cast<long>(rows_per_thread) * groups < dim || !raw)
+        parts <= 0 || slice <= 0 || slice > vdim || rot < 0 || rot % 2 || rot > dim ||
+        (rot > 0 && (!cos_table || !sin_table)) || !(eps > 0.f) ||
+        static_cast<long>(rows_per_thread) * groups * parts < dim || !raw || !turned)
         return CIE_BAD_ARGUMENT;
     const int slices = (vdim + slice - 1) / slice;
     const int threads = ((slice * groups + kWave - 1) / kWave) * kWave;
+    const int rows = groups * rows_per_thread;
+    const int padded = rows * parts;
     const size_t lds = sizeof(float) * static_cast<size_t>(chunk) *
-                       (2 * static_cast<size_t>(groups) * rows_per_thread + slice + static_cast<size_t>(groups) * slice);
-    if (threads > 1024 || lds > 64 * 1024 || slices > 65535) return CIE_BAD_ARGUMENT;
+                       (2 * static_cast<size_t>(rows) + slice + static_cast<size_t>(groups) * slice);
+    if (threads > 512 || lds > 64 * 1024 || static_cast<long>(slices) * parts > 65535 ||
+        static_cast<long>(chunk) * 2 * rows / 4 > static_cast<long>(kFetchPieces) * threads ||
+        static_cast<long>(chunk) * slice > static_cast<long>(kFetchValues) * threads)
+        return CIE_BAD_ARGUMENT;
     if (sequences == 0 || tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    dim3 grid(sequences, heads, slices);
+    if (dtype == CIE_F32)
+        retention_turn_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(proj), ldp, q_off, k_off, cos_table,
+                                                           sin_table, rot, positions, turned, heads, dim, padded, key_scale);
+    else if (dtype == CIE_BF16)
+        retention_turn_kernel<bf16_t><<<tokens, 256, 0, s>>>(static_cast<const bf16_t*>(proj), ldp, q_off, k_off, cos_table,
+                                                            sin_table, rot, positions, turned, heads, dim, padded, key_scale);
+    else
+        return CIE_BAD_ARGUMENT;
+    dim3 grid(sequences, heads, slices * parts);
+    const long plane = static_cast<long>(tokens) * heads * vdim;
     int code = CIE_BAD_ARGUMENT;
-#define CIE_RETENTION(T, DS)                                                                                          \
-    code = launch_retention<T, DS>(s, grid, threads, lds, proj, ldp, q_off, k_off, v_off, cos_table, sin_table, rot,  \
-                                   decay, state, seq_slot, seq_start, q_start_loc, raw, heads, dim, vdim, slice,      \
-                                   groups, chunk, key_scale)
+#define CIE_RETENTION(T, DS)                                                                                         \
+    code = launch_retention<T, DS>(s, grid, threads, lds, proj, ldp, v_off, turned, decay, state, seq_slot,          \
+                                   q_start_loc, raw, plane, heads, dim, vdim, slice, slices, groups, padded, chunk)
     if (dtype == CIE_F32) {
         if (rows_per_thread == 4) CIE_RETENTION(float, 4);
         else if (rows_per_thread == 8) CIE_RETENTION(float, 8);
         else if (rows_per_thread == 16) CIE_RETENTION(float, 16);
         else if (rows_per_thread == 32) CIE_RETENTION(float, 32);
-    } else if (dtype == CIE_BF16) {
+    } else {
         if (rows_per_thread == 4) CIE_RETENTION(bf16_t, 4);
         else if (rows_per_thread == 8) CIE_RETENTION(bf16_t, 8);
         else if (rows_per_thread == 16) CIE_RETENTION(bf16_t, 16);
@@ -315,10 +413,10 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     const int items = tokens * heads;
     const int blocks = (items + 3) / 4;
     if (dtype == CIE_F32)
-        retention_norm_kernel<float><<<blocks, 256, 0, s>>>(raw, static_cast<const float*>(proj), ldp, g_off,
+        retention_norm_kernel<float><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const float*>(proj), ldp, g_off,
                                                            static_cast<float*>(out), tokens, heads, vdim, eps);
     else
-        retention_norm_kernel<bf16_t><<<blocks, 256, 0, s>>>(raw, static_cast<const bf16_t*>(proj), ldp, g_off,
+        retention_norm_kernel<bf16_t><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const bf16_t*>(proj), ldp, g_off,
                                                             static_cast<bf16_t*>(out), tokens, heads, vdim, eps);
     return cie_after_launch();
 }
@@ -352,16 +450,15 @@ CIE_API int cie_gated_recurrence(void* stream, int dtype, const void* y_pre, lon
         return CIE_BAD_ARGUMENT;
     if (sequences == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    dim3 grid((channels + kScanChannels - 1) / kScanChannels, sequences);
-    const int threads = kScanChannels * segments;
-    if (dtype == CIE_F32)
-        gated_recurrence_kernel<float><<<grid, threads, 0, s>>>(
-            static_cast<const float*>(y_pre), ldy, static_cast<const float*>(x_in), ldx, static_cast<const float*>(u), gates,
-            block_width, rate, state, past, seq_slot, q_start_loc, static_cast<float*>(out), channels, taps, segments);
-    else if (dtype == CIE_BF16)
-        gated_recurrence_kernel<bf16_t><<<grid, threads, 0, s>>>(
-            static_cast<const bf16_t*>(y_pre), ldy, static_cast<const bf16_t*>(x_in), ldx, static_cast<const bf16_t*>(u),
-            gates, block_width, rate, state, past, seq_slot, q_start_loc, static_cast<bf16_t*>(out), channels, taps, segments);
+#define CIE_SCAN(T, CH)                                                                                             \
+    gated_recurrence_kernel<T, CH><<<dim3((channels + CH - 1) / CH, sequences), CH * segments, 0, s>>>(               \
+        static_cast<const T*>(y_pre), ldy, static_cast<const T*>(x_in), ldx, static_cast<const T*>(u), gates,          \
+        block_width, rate, state, past, seq_slot, q_start_loc, static_cast<T*>(out), channels, taps, segments)
+    if (dtype == CIE_F32 && segments == 1) CIE_SCAN(float, 64);
+    else if (dtype == CIE_F32) CIE_SCAN(float, 16);
+    else if (dtype == CIE_BF16 && segments == 1) CIE_SCAN(bf16_t, 64);
+    else if (dtype == CIE_BF16) CIE_SCAN(bf16_t, 16);
+#undef CIE_SCAN
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

@@ -926,30 +926,41 @@ RETENTION_SLICE = 64             # value columns of a head that one workgroup ta
 RETENTION_LDS_FLOATS = 15 * 1024
 
 
-def plan_retention(dim: int, vdim: int) -> tuple[int, int, int, int]:
-    """(rows per thread, groups of threads, value columns per workgroup, tokens per chunk) of the retention kernel
-    for heads of ``dim`` x ``vdim``: workgroups of up to 512 threads where the rows allow it (1,024 otherwise)."""
-    if dim < 1 or vdim < 1:
+def plan_retention(dim: int, vdim: int, units: int = 1) -> tuple[int, int, int, int, int]:
+    """(rows per thread, groups of threads, parts of the rows, value columns per workgroup, tokens per chunk) of
+    the retention kernel for heads of ``dim`` x ``vdim`` when ``units`` (sequence, head) pairs run: a workgroup takes
+    up to 64 value columns and a part of a head's rows, as many parts as give every compute unit a workgroup;
+    workgroups of up to 512 threads."""
+    if dim < 1 or vdim < 1 or units < 1:
         raise ValueError("head sizes must be positive")
     piece = min(vdim, RETENTION_SLICE)
-    rows = next((r for r in RETENTION_ROWS if -(-dim // r) * piece <= 512), None)
-    if rows is None:
-        rows = next((r for r in RETENTION_ROWS if -(-dim // r) * piece <= 1024), None)
+    slices = -(-vdim // piece)
+    most_groups = max(1, 512 // (-(-piece // 8) * 8))
+    parts = max(1, min(compute_units() // (units * slices), -(-dim // 4)))
+    parts = max(parts, -(-dim // (most_groups * RETENTION_ROWS[-1])))  # (no more rows than a workgroup can keep)
+    share = -(-dim // parts)  # rows of a part
+    rows = next((r for r in RETENTION_ROWS if -(-share // r) <= most_groups), None)
     if rows is None:
         raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's registers")
-    groups = -(-dim // rows)
+    groups = -(-share // rows)
+    parts = -(-dim // (groups * rows))
     per_token = 2 * groups * rows + piece + groups * piece
-    chunk = min(32, RETENTION_LDS_FLOATS // per_token)
-    if chunk < 1:
+    threads = -(-piece * groups // 64) * 64
+    # (what a chunk holds must fit the LDS, and what a thread fetches ahead of a chunk its registers:
+    # six 16-byte pieces of queries and keys and twelve values).  Long chunks: the next chunk's numbers are on
+    # their way from memory for as long as the walk over the current one takes.
+    chunk = min(48, RETENTION_LDS_FLOATS // per_token, 6 * threads * 4 // (2 * groups * rows), 12 * threads // piece)
+    if chunk < 1 or threads > 512:
         raise ValueError(f"heads of {dim} x {vdim} do not fit the retention kernel's LDS")
-    return rows, groups, piece, chunk
+    return rows, groups, parts, piece, chunk
 
 
 def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optional[torch.Tensor],
               sin: Optional[torch.Tensor], rot: int, decay: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
-              seq_start: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int, dim: int, vdim: int,
+              positions: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int, dim: int, vdim: int,
               eps: float, key_scale: float, longest_position: int) -> torch.Tensor:
-    """Retention over a step's tokens (``csrc/recurrent.hip``).  ``proj`` [T, ...] holds each token's queries, keys
+    """Retention over a step's tokens (``csrc/recurrent.hip``; ``positions`` int32 [T] are the tokens' own).
+    ``proj`` [T, ...] holds each token's queries, keys
     (heads x dim), values and gates (heads x vdim) from the columns ``offsets`` on; ``state`` float32
     [slots, heads, dim, vdim] is read and written at the sequences' slots; cos/sin float32 [positions, rot/2]
     must reach ``longest_position``.  Returns [T, heads * vdim] in ``proj``'s type."""
@@ -968,20 +979,21 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
     _gpu("state", state, torch.float32, 4)
     if decay.shape[0] != heads or tuple(state.shape[1:]) != (heads, dim, vdim):
         raise ValueError(f"decay {tuple(decay.shape)} / state {tuple(state.shape)} do not fit {heads} heads of {dim} x {vdim}")
-    for name, meta, least in (("seq_slot", seq_slot, sequences), ("seq_start", seq_start, sequences),
+    for name, meta, least in (("seq_slot", seq_slot, sequences), ("positions", positions, tokens),
                               ("q_start_loc", q_start_loc, sequences + 1)):
         _gpu(name, meta, torch.int32, 1)
         if meta.shape[0] < least:
-            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
-    rows, groups, piece, chunk = plan_retention(dim, vdim)
-    raw = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+            raise ValueError(f"{name} has {meta.shape[0]} entries, {least} are needed")
+    rows, groups, parts, piece, chunk = plan_retention(dim, vdim, max(1, sequences * heads))
+    turned = torch.empty((tokens, heads, 2, parts * groups * rows), dtype=torch.float32, device=proj.device)
+    raw = torch.empty((parts, tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
     ldp = proj.stride(0) if tokens > 1 else max(proj.stride(0), proj.shape[1])
     _run("cie_retention", load_library().cie_retention(
         _stream(), _i(_code(proj.dtype)), _ptr(proj), ldp, _i(q_off), _i(k_off), _i(v_off), _i(g_off),
         _ptr(cos if rot else None), _ptr(sin if rot else None), _i(rot), _ptr(decay), _ptr(state), _ptr(seq_slot),
-        _ptr(seq_start), _ptr(q_start_loc), _ptr(raw), _ptr(out), _i(tokens), _i(sequences), _i(heads), _i(dim), _i(vdim),
-        _i(rows), _i(groups), _i(piece), _i(chunk), _f(eps), _f(key_scale)))
+        _ptr(positions), _ptr(q_start_loc), _ptr(turned), _ptr(raw), _ptr(out), _i(tokens), _i(sequences), _i(heads), _i(dim), _i(vdim),
+        _i(rows), _i(groups), _i(parts), _i(piece), _i(chunk), _f(eps), _f(key_scale)))
     return out
 
 

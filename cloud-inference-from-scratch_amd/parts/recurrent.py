@@ -82,7 +82,7 @@ class Retention(Part):
         cos, sin = self.position.tables(x.device, bound) if rot else (None, None)
         proj = linear(x, self.w_in)
         out = ops.retention(proj, (0, h * d, 2 * h * d, 2 * h * d + h * v), cos, sin, rot, self.decay, view.state,
-                            batch.seq_slot, batch.seq_start, batch.q_start_loc, batch.sequences, h, d, v, self.eps,
+                            batch.seq_slot, batch.positions, batch.q_start_loc, batch.sequences, h, d, v, self.eps,
                             d ** -0.5, bound - 1)
         return linear(out, self.w_o)
 

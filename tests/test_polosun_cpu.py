@@ -194,9 +194,11 @@ def test_plain_model_composes_branches_and_depth_average():
 def test_retention_kernel_plan_fits_its_limits():
     from cie_amd.kernels import ops
 
-    for dim, vdim in ((32, 64), (8, 40), (128, 256), (256, 64), (4, 72), (32, 1024), (512, 512), (3, 5)):
-        rows, groups, piece, chunk = ops.plan_retention(dim, vdim)
-        assert rows in ops.RETENTION_ROWS and rows * groups >= dim and piece * groups <= 1024 and piece <= min(vdim, 64)
-        assert chunk >= 1 and chunk * (2 * rows * groups + piece + groups * piece) <= ops.RETENTION_LDS_FLOATS
-    with pytest.raises(ValueError):
-        ops.plan_retention(1024, 64)
+    for dim, vdim in ((32, 64), (8, 40), (128, 256), (256, 64), (4, 72), (32, 1024), (512, 512), (3, 5), (1024, 64)):
+        for units in (1, 8, 64, 1000):
+            rows, groups, parts, piece, chunk = ops.plan_retention(dim, vdim, units)
+            assert rows in ops.RETENTION_ROWS and rows * groups * parts >= dim and piece <= min(vdim, 64)
+            threads = -(-piece * groups // 64) * 64
+            assert threads <= 512 and (parts - 1) * rows * groups < dim
+            assert chunk >= 1 and chunk * (2 * rows * groups + piece + groups * piece) <= ops.RETENTION_LDS_FLOATS
+            assert chunk * 2 * rows * groups // 4 <= 6 * threads and chunk * piece <= 12 * threads
