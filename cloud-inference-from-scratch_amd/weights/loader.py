@@ -195,7 +195,8 @@ class RandomSource:
             spec = expected[name]
             return self.draw(place[name], spec).to(_target_dtype(spec, torch.bfloat16, target)).to(device)
 
-        return TensorsOnDemand(expected, make)
+        # (a tensor that a checkpoint may hold but the model does not read is not drawn)
+        return TensorsOnDemand([name for name, spec in expected.items() if not spec.optional], make)
 
     def load(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
              tied_optional: Mapping[str, str] | None = None) -> dict[str, torch.Tensor]:

@@ -202,3 +202,22 @@ def test_retention_kernel_plan_fits_its_limits():
             assert threads <= 512 and (parts - 1) * rows * groups < dim
             assert chunk >= 1 and chunk * (2 * rows * groups + piece + groups * piece) <= ops.RETENTION_LDS_FLOATS
             assert chunk * 2 * rows * groups // 4 <= 6 * threads and chunk * piece <= 12 * threads
+
+
+def test_the_command_line_writes_a_model_folder_of_this_design(tmp_path, capsys):
+    import json
+
+    from cie_amd import cli
+    from cie_amd.config import load_config
+
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(pu.SMALL_B))
+    assert cli.main(["init-model", "--config", str(config_file), "--out", str(tmp_path / "model"), "--seed", "3"]) == 0
+    assert load_config(tmp_path / "model").to_hf_config()["layers"][2]["type"] == "latent_attention"
+    from safetensors import safe_open
+
+    with safe_open(str(tmp_path / "model" / "model.safetensors"), framework="pt") as handle:
+        names = set(handle.keys())
+    assert "l2.mix.dkv.norm" in names and "l2.norm2" not in names and "l1.norm2" in names
+    assert cli.main(["models"]) == 0
+    assert "Polosun" in capsys.readouterr().out
