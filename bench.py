@@ -242,7 +242,7 @@ def polosun_raw(shape: dict, layers: int) -> dict:
         {"type": "latent_attention", "mlp": mlp,
          "mixer": {"heads": width // 128, "dim": 128, "rot_dim": 32, "vdim": 128, "kv_rank": 96, "scale": 160 ** -0.5,
                    "rot": {"base": 1000000.0, "dims": 32,
-                           "scaling": {"factor": 8.0, "fast": 32.0, "original": 4096, "slow": 1.0}}}},
+                           "scaling": {"factor": 4.0, "fast": 32.0, "original": 8192, "slow": 1.0}}}},
         {"type": "rglru", "mlp": mlp, "mixer": {"width": width, "blocks": width // 256, "conv": 4}},
     ]
     return {"architecture": "Polosun", "vocab": shape["vocab_size"], "width": width, "residual_mult": 0.5,
