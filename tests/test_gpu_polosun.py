@@ -300,3 +300,69 @@ def test_the_trace_runner_replays_a_model_folder(tmp_path, models):
                for s in steps if any(e["want"] for e in s["entries"])}
     worst, _ = pu.spread(replay_util.by_position(steps, outputs), plain)
     assert worst <= LIMIT["float32"], worst
+
+
+# ---------------------------------------------------------------- kernels alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [1, 7, 16, 17, 64, 150])
+def test_block_diagonal_product_in_all_its_forms(rows, dtype):
+    """Few rows, tiles, and (bfloat16) the matrix cores; blocks read from and written to columns of wider rows, with
+    bias, with a sigmoid gate, float32 results from bfloat16 operands; a K that is no multiple of 32, and one that is
+    no multiple of 8 (which keeps off the matrix cores)."""
+    from cie_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(rows)
+    for blocks, n, k, a_block, extra in ((3, 24, 40, 56, 8), (2, 80, 96, 96, 0), (5, 17, 12, 20, 4)):
+        a = torch.randn(rows, extra + (blocks - 1) * a_block + k + 3, generator=g).to(dtype).cuda()
+        w = (torch.randn(blocks, n, k, generator=g) / k ** 0.5).to(dtype).cuda()
+        bias = torch.randn(blocks, n, generator=g).to(dtype).cuda()
+        gate = torch.randn(rows, 5 + blocks * n, generator=g).to(dtype).cuda()
+        picked = torch.stack([a[:, extra + b * a_block: extra + b * a_block + k] for b in range(blocks)], 1).double()
+        plain = torch.einsum("mbk,bnk->mbn", picked, w.double())
+        tol = 2e-5 if dtype == torch.float32 else 2e-2
+        out = ops.block_linear(a, w, a_block=a_block, a_offset=extra, out_dtype=torch.float32)
+        assert torch.allclose(out.double().reshape(rows, blocks, n), plain, atol=2e-5 if dtype == torch.float32 else 1e-4)
+        with_bias = ops.block_linear(a, w, bias, a_block=a_block, a_offset=extra)
+        assert with_bias.dtype == dtype
+        assert torch.allclose(with_bias.double().reshape(rows, blocks, n), plain + bias.double(), atol=tol, rtol=tol)
+        wide = torch.full((rows, 6 + blocks * (n + 2)), 7.0, dtype=dtype, device="cuda")
+        ops.block_linear(a, w, a_block=a_block, a_offset=extra, out=wide, out_offset=6, c_block=n + 2, gate=gate, gate_offset=5)
+        gated = plain * torch.sigmoid(gate[:, 5:].double().reshape(rows, blocks, n))
+        got = wide[:, 6:].reshape(rows, blocks, n + 2)
+        assert torch.allclose(got[:, :, :n].double(), gated, atol=tol, rtol=tol)
+        assert bool((wide[:, :6] == 7).all()) and bool((got[:, :-1, n:] == 7).all())  # nothing beside the blocks is touched
+    # a row's result does not depend on the rows beside it
+    if rows > 1:
+        alone = ops.block_linear(a[:1].contiguous(), w, a_block=a_block, a_offset=extra, out_dtype=torch.float32)
+        if (rows <= 16) == (1 <= 16):
+            assert torch.equal(alone, out[:1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layer_boundary_kernel(dtype):
+    from cie_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(1)
+    for rows, hidden in ((3, 40), (130, 1024), (9, 2048)):
+        history = torch.randn(5, rows, hidden, generator=g).cuda()
+        x = torch.randn(rows, hidden, generator=g).cuda()
+        a = torch.randn(rows, hidden, generator=g).to(dtype).cuda()
+        b = torch.randn(rows, hidden, generator=g).to(dtype).cuda()
+        weights = torch.randn(4, generator=g).cuda()
+        kept = history.clone()
+        stream, normed = ops.depth_stream(x, a, b, mult=0.7, history=history, newest=3, weights=weights, gains=(1.5, 0.25),
+                                          out_dtype=dtype, eps=1e-5)
+        new = x.double() + 0.7 * (a.double() + b.double())
+        assert torch.allclose(history[3].double(), new, atol=1e-5) and torch.equal(history[[0, 1, 2, 4]], kept[[0, 1, 2, 4]])
+        want = sum(weights[j].double() * (new if j == 3 else kept[j].double()) for j in range(4))
+        assert torch.allclose(stream.double(), want, atol=2e-5)
+        unit = want / torch.sqrt((want * want).mean(-1, keepdim=True) + 1e-5)
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        assert torch.allclose(normed[0].double(), unit * 1.5, atol=tol, rtol=tol)
+        assert torch.allclose(normed[1].double(), unit * 0.25, atol=tol, rtol=tol)
+        # one branch, no average, one norm; and norms alone
+        stream, normed = ops.depth_stream(x, a, mult=2.0, gains=(1.0,), out_dtype=dtype, eps=1e-5)
+        assert torch.allclose(stream.double(), x.double() + 2.0 * a.double(), atol=1e-5) and len(normed) == 1
+        nothing, normed = ops.depth_stream(x, gains=(3.0, 1.0), out_dtype=dtype, eps=1e-5, want_stream=False)
+        unit = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5)
+        assert nothing is None and torch.allclose(normed[0].double(), 3.0 * unit, atol=tol, rtol=tol)
