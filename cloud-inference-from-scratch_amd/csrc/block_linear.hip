@@ -12,7 +12,7 @@
 // of k (blocks of 256 summed, then the blocks' sums), so a row's result does not depend on the other rows; the
 // result is float32 or the operands' type.  64 x 64 results per workgroup, slices of 16 k through LDS; up to 16 rows
 // take a form of their own (below) whose sums have another fixed order, again the same for every row, and bfloat16
-// operands with more rows go to the matrix cores (further below) where their addresses allow 16-byte loads.
+// operands of more than four rows go to the matrix cores (further below) where their addresses allow 16-byte loads.
 #include "common.h"
 
 namespace {
@@ -156,7 +156,7 @@ int launch_rows(hipStream_t s, const void* A, long lda, long a_block, const void
 #undef CIE_ROWS
     return cie_after_launch();
 }
-// bfloat16 operands with more rows than that: the matrix cores.  A wave owns 16 result columns and up to four tiles
+// bfloat16 operands with more than four rows: the matrix cores.  A wave owns 16 result columns and up to four tiles
 // of 16 rows; a workgroup's four waves take 64 columns side by side.  Per slice of 32 k a lane loads the 8 numbers of
 // its weight row (column n0 + lane % 16, k from 8 * (lane / 16)) and of its row of A in each tile as 16 bytes, which
 // is the operand layout of v_mfma_f32_16x16x32_bf16 as it is; the rows of A come through the cache (the weights of a
@@ -235,14 +235,17 @@ CIE_API int cie_block_linear(void* stream, int dtype, int out_f32, const void* A
     if (grid_y > 65535) return CIE_BAD_ARGUMENT;
     dim3 grid((N + TN - 1) / TN, grid_y, B);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (M <= kRowsMost) {
+    const bool cores = dtype == CIE_BF16 && K % 8 == 0 && lda % 8 == 0 && a_block % 8 == 0 &&
+                       reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+    // (measured at the 3B widths, a decode step of 12 layers: 8 rows 1.26 ms in the few-row form, 1.19 ms on the matrix
+    // cores; one row 1.08 against 1.10)
+    if (M <= kRowsMost && !(cores && M > 4)) {
         if (dtype == CIE_F32) return launch_rows<float, float>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
         if (dtype == CIE_BF16 && out_f32) return launch_rows<bf16_t, float>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
         if (dtype == CIE_BF16) return launch_rows<bf16_t, bf16_t>(s, A, lda, a_block, W, bias, C, ldc, c_block, gate, ldg, g_block, M, N, K, B);
         return CIE_BAD_ARGUMENT;
     }
-    if (dtype == CIE_BF16 && K % 8 == 0 && lda % 8 == 0 && a_block % 8 == 0 &&
-        reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0) {
+    if (cores) {
         dim3 tiles((N + 63) / 64, grid_y, B);
         if (out_f32)
             block_linear_mfma_kernel<float><<<tiles, 256, 0, s>>>(

@@ -332,10 +332,9 @@ def test_block_diagonal_product_in_all_its_forms(rows, dtype):
         assert torch.allclose(got[:, :, :n].double(), gated, atol=tol, rtol=tol)
         assert bool((wide[:, :6] == 7).all()) and bool((got[:, :-1, n:] == 7).all())  # nothing beside the blocks is touched
     # a row's result does not depend on the rows beside it
-    if rows > 1:
+    if 1 < rows <= 4 or (dtype == torch.float32 and rows <= 16):  # (within one form of the kernel, bit for bit)
         alone = ops.block_linear(a[:1].contiguous(), w, a_block=a_block, a_offset=extra, out_dtype=torch.float32)
-        if (rows <= 16) == (1 <= 16):
-            assert torch.equal(alone, out[:1])
+        assert torch.equal(alone, out[:1])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
