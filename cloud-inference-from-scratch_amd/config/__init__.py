@@ -1,4 +1,5 @@
 from .engine_config import EngineConfig, build_engine_config, canonical_dtype
+from .givizen import GivizenConfig
 from .polosun import PolosunConfig
 from .qwen2 import Qwen2Config
 from .registry import (
@@ -14,9 +15,10 @@ from .specs import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec
 # the architectures this package brings; others register themselves the same way from outside
 register_architecture("Qwen2ForCausalLM", Qwen2Config, model_type="qwen2")
 register_architecture("Polosun", PolosunConfig)
+register_architecture("Givizen", GivizenConfig)
 
 __all__ = [
-    "ARCHITECTURES", "Architecture", "ConfigError", "EngineConfig", "LayerCall", "LayerSpec",
+    "ARCHITECTURES", "Architecture", "ConfigError", "EngineConfig", "GivizenConfig", "LayerCall", "LayerSpec",
     "ModelSpec", "PartSpec", "PolosunConfig", "Qwen2Config", "architecture_of", "build_engine_config",
     "canonical_dtype", "config_from_dict", "load_config", "register_architecture",
 ]

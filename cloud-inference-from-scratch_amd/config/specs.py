@@ -91,6 +91,8 @@ class ModelSpec:
     final_norm_name: str = "model.norm"
     head_name: str = "lm_head.weight"
     layer_prefix: str = "model.layers.{index}."
+    embedding_scale: float = 1.0          # the embedding's rows are multiplied by this on their way into the stream
+    logit_softcap: float | None = None    # logits <- cap * tanh(logits / cap)
     extra: dict[str, Any] = field(default_factory=dict, compare=False)
 
     def __post_init__(self) -> None:

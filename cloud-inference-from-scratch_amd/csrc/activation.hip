@@ -3,6 +3,7 @@
 // With `row_sumsq` the rows of gate_up come from a product whose input rows lacked the 1/rms of an
 // RMSNorm (a product is linear in its rows): both halves are first multiplied by
 // rsqrt(sum of the row's `parts` partial sums of squares / hidden + eps).
+#include "activation_forms.h"
 #include "common.h"
 
 // the row's factor, made by the whole workgroup; 1 without row_sumsq
@@ -73,5 +74,47 @@ CIE_API int cie_silu_mul(void* stream, int dtype, const void* gate_up, void* out
                                                     row_sumsq, parts, hidden, eps);
     else
         return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// The gated unit with bounded inputs (activation_forms.h) over rows [tokens, 2 * intermediate], gate half first.
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int intermediate, float limit,
+                                   float alpha, float offset) {
+    const int token = blockIdx.x;
+    const int i = blockIdx.y * blockDim.x + threadIdx.x;
+    if (i >= intermediate) return;
+    const T* row = gate_up + static_cast<size_t>(token) * 2 * intermediate;
+    out[static_cast<size_t>(token) * intermediate + i] =
+        from_float<T>(clamped_glu(to_float(row[i]), to_float(row[intermediate + i]), limit, alpha, offset));
+}
+
+CIE_API int cie_clamped_glu(void* stream, int dtype, const void* gate_up, void* out, int tokens, int intermediate,
+                            float limit, float alpha, float offset) {
+    if (tokens < 0 || intermediate <= 0 || (intermediate + 255) / 256 > 65535 || !(limit > 0.f)) return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid(tokens, (intermediate + 255) / 256);
+    if (dtype == CIE_F32)
+        clamped_glu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out),
+                                                      intermediate, limit, alpha, offset);
+    else if (dtype == CIE_BF16)
+        clamped_glu_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
+                                                       intermediate, limit, alpha, offset);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// A smooth bound on float32 values, in place: x <- cap * tanh(x / cap).
+__global__ void soft_cap_kernel(float* __restrict__ x, long count, float cap) {
+    const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) x[i] = cap * tanhf(x[i] / cap);
+}
+
+CIE_API int cie_soft_cap(void* stream, float* x, long count, float cap) {
+    if (count < 0 || !(cap > 0.f) || (count + 255) / 256 > 0x7fffffffL) return CIE_BAD_ARGUMENT;
+    if (count == 0) return CIE_OK;
+    soft_cap_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(x, count, cap);
     return cie_after_launch();
 }

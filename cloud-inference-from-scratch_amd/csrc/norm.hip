@@ -148,3 +148,62 @@ CIE_API int cie_add_rmsnorm(void* stream, int dtype, int wdtype, float* residual
         return launch_norm<bf16_t, float>(s, residual, branch, weight, out, rows, n_out, hidden, eps, write_residual);
     return CIE_BAD_ARGUMENT;
 }
+
+// Norm on a branch's output, then the add:  y = branch[row] (+ the sum of `parts` float32 rows [tokens, parts, hidden]);
+//   residual[row] += y / sqrt(mean(y^2) + eps) * weight
+// (the weight as it multiplies: a weight stored around zero comes here with the one added).  With `rows_out`
+// the new stream is also written in the activation type, for the products of the sublayer that reads it next.
+// Statistics, scaling and the sum are float32.  One workgroup per row, the row staged in LDS.
+template <typename B, typename T>
+__global__ void branch_norm_add_kernel(float* __restrict__ residual, const B* __restrict__ branch,
+                                       const float* __restrict__ parts, int n_parts,
+                                       const float* __restrict__ weight, T* __restrict__ rows_out, int hidden,
+                                       float eps) {
+    extern __shared__ float staged[];
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    const B* add = branch ? branch + row * hidden : nullptr;
+    const float* extra = parts ? parts + row * n_parts * hidden : nullptr;
+    float sum_sq = 0.f;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+        float y = add ? to_float(add[h]) : 0.f;
+        for (int p = 0; p < n_parts; ++p) y += extra[static_cast<size_t>(p) * hidden + h];
+        staged[h] = y;
+        sum_sq += y * y;
+    }
+    const float total = block_sum(sum_sq, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    float* res = residual + row * hidden;
+    T* dst = rows_out ? rows_out + row * hidden : nullptr;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+        const float x = res[h] + (staged[h] * inv) * weight[h];
+        res[h] = x;
+        if (dst) dst[h] = from_float<T>(x);
+    }
+}
+
+// bdtype: storage type of `branch` (ignored without one); dtype: type of rows_out.
+CIE_API int cie_branch_norm_add(void* stream, int bdtype, int dtype, float* residual, const void* branch,
+                                const float* parts, int n_parts, const float* weight, void* rows_out, int tokens,
+                                int hidden, float eps) {
+    if (tokens < 0 || hidden <= 0 || hidden * sizeof(float) > 64 * 1024 || !(eps > 0.f) || n_parts < 0 ||
+        (n_parts > 0 && !parts) || (!branch && n_parts == 0))
+        return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int threads = tokens <= 64 ? 1024 : 256;
+    const size_t lds = hidden * sizeof(float);
+    if (!parts) n_parts = 0;
+    if (dtype == CIE_F32 && (bdtype == CIE_F32 || !branch))
+        branch_norm_add_kernel<float, float><<<tokens, threads, lds, s>>>(
+            residual, static_cast<const float*>(branch), parts, n_parts, weight, static_cast<float*>(rows_out), hidden, eps);
+    else if (dtype == CIE_BF16 && bdtype == CIE_BF16)
+        branch_norm_add_kernel<bf16_t, bf16_t><<<tokens, threads, lds, s>>>(
+            residual, static_cast<const bf16_t*>(branch), parts, n_parts, weight, static_cast<bf16_t*>(rows_out), hidden, eps);
+    else if (dtype == CIE_BF16 && bdtype == CIE_F32)
+        branch_norm_add_kernel<float, bf16_t><<<tokens, threads, lds, s>>>(
+            residual, static_cast<const float*>(branch), parts, n_parts, weight, static_cast<bf16_t*>(rows_out), hidden, eps);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

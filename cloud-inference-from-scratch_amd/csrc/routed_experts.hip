@@ -1,0 +1,369 @@
+// A feed-forward of many small gated experts of which every token uses a few.
+//
+//   route      s = sigmoid(z) for float32 router logits z [tokens, experts]; the `top` largest are chosen (the
+//              lowest index wins a tie); a (token, choice) *pair* p = token * top + k gets the expert and the
+//              score as it is (not renormalised).
+//   arrange    pairs sorted by expert and cut into tiles of at most `tile_rows` rows of one expert; everything the
+//              later kernels need stays on the device (the count of tiles too), so a step can be captured: grids
+//              are sized for the most tiles there can be, and workgroups past the count leave at once.
+//   gate_up    act[i, :] = glu(W_gate[e] (w x), W_up[e] (w x)) for the i-th sorted pair: the pair's weight w
+//              multiplies the expert's *input* row x (the unit is not linear, so it cannot move to the output).
+//   down       parts[p, :] = W_down[e] act[i, :], float32, one row per pair: whoever adds the branch sums a
+//              token's `top` rows, in a fixed order.
+//
+// bfloat16 with widths that are multiples of 8 runs on the matrix cores (four waves a workgroup, each a tile of 16
+// columns over all of K for up to 16 * RT rows); anything else takes the plain form of one thread per result, whose
+// sums run over k in order, float32.  Weights: gate_up [experts, 2 * ff, hidden] (gate rows first), down
+// [experts, hidden, ff].
+#include "activation_forms.h"
+#include "attention_args.h"
+#include "common.h"
+
+using cie_attention::bf16x8;
+using cie_attention::floatx4;
+
+namespace {
+
+constexpr int kMaxExperts = 1024;
+
+// One wave per token.
+__global__ void __launch_bounds__(256)
+route_kernel(const float* __restrict__ logits, int tokens, int experts, int top, int* __restrict__ pair_expert,
+             float* __restrict__ pair_weight) {
+    const int lane = threadIdx.x % kWave;
+    const int token = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (token >= tokens) return;
+    const float* z = logits + static_cast<size_t>(token) * experts;
+    constexpr int kMine = kMaxExperts / kWave;
+    float mine[kMine];
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+        const int e = lane + i * kWave;
+        mine[i] = e < experts ? 1.0f / (1.0f + expf(-z[e])) : -1.f;  // (scores lie in [0, 1]; -1: no such expert)
+    }
+    for (int k = 0; k < top; ++k) {
+        float best = -2.f;
+        int best_e = kMaxExperts;
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            if (mine[i] > best) {  // (ascending index within the lane: the first of equals stays)
+                best = mine[i];
+                best_e = lane + i * kWave;
+            }
+        }
+#pragma unroll
+        for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+            const float other = __shfl_xor(best, offset, kWave);
+            const int other_e = __shfl_xor(best_e, offset, kWave);
+            if (other > best || (other == best && other_e < best_e)) {
+                best = other;
+                best_e = other_e;
+            }
+        }
+        if (lane == 0) {
+            pair_expert[static_cast<size_t>(token) * top + k] = best_e;
+            pair_weight[static_cast<size_t>(token) * top + k] = best;
+        }
+#pragma unroll
+        for (int i = 0; i < kMine; ++i)
+            if (lane + i * kWave == best_e) mine[i] = -3.f;
+    }
+}
+
+// One workgroup.  sorted[i]: the pair at place i of the order by expert; tiles (expert, first place, rows).
+__global__ void __launch_bounds__(1024)
+arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int tile_rows, int* __restrict__ sorted,
+               int* __restrict__ tile_expert, int* __restrict__ tile_begin, int* __restrict__ tile_count,
+               int* __restrict__ n_tiles) {
+    __shared__ int count[kMaxExperts];
+    __shared__ int first[kMaxExperts];
+    __shared__ int first_tile[kMaxExperts];
+    __shared__ int cursor[kMaxExperts];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+        count[e] = 0;
+        cursor[e] = 0;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[pair_expert[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int place = 0, tile = 0;
+        for (int e = 0; e < experts; ++e) {
+            first[e] = place;
+            first_tile[e] = tile;
+            place += count[e];
+            tile += (count[e] + tile_rows - 1) / tile_rows;
+        }
+        *n_tiles = tile;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+        const int tiles = (count[e] + tile_rows - 1) / tile_rows;
+        for (int t = 0; t < tiles; ++t) {
+            tile_expert[first_tile[e] + t] = e;
+            tile_begin[first_tile[e] + t] = first[e] + t * tile_rows;
+            tile_count[first_tile[e] + t] = min(tile_rows, count[e] - t * tile_rows);
+        }
+    }
+    // (the order of an expert's pairs among themselves follows the order of arrival: every row is computed
+    //  by itself, so no result depends on it)
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = pair_expert[p];
+        sorted[first[e] + atomicAdd(&cursor[e], 1)] = p;
+    }
+}
+
+struct ExpertArgs {
+    const int* sorted;
+    const float* pair_weight;
+    const int* tile_expert;
+    const int* tile_begin;
+    const int* tile_count;
+    const int* n_tiles;
+    int top;
+    int hidden;
+    int ff;
+    float limit;
+    float alpha;
+    float offset;
+};
+
+__device__ __forceinline__ bf16x8 scaled_fragment(const uint4 raw, float w) {
+    const uint32_t v[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        out[i] = pack_bf16(__uint_as_float(v[i] << 16) * w, __uint_as_float(v[i] & 0xffff0000u) * w);
+    return __builtin_bit_cast(bf16x8, (uint4{out[0], out[1], out[2], out[3]}));
+}
+
+// v_mfma_f32_16x16x32_bf16 with A = rows of x (lane % 16 the row, lane / 16 the eighth of the 32 k), B = rows of
+// the weight (lane % 16 the result column, the same k): lane (r, g) then holds the results of rows g*4 .. g*4+3 at
+// column r.
+template <int RT>
+__global__ void __launch_bounds__(256)
+experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_gate_up,
+                            bf16_t* __restrict__ act, ExpertArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= *a.n_tiles) return;
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int c0 = (blockIdx.y * 4 + wave) * 16;
+    if (c0 >= a.ff) return;
+    const int expert = a.tile_expert[tile];
+    const int begin = a.tile_begin[tile];
+    const int rows = a.tile_count[tile];
+    const int K = a.hidden;
+    const bool col_ok = c0 + r < a.ff;
+    const bf16_t* wg = w_gate_up + (static_cast<size_t>(expert) * 2 * a.ff + min(c0 + r, a.ff - 1)) * K;
+    const bf16_t* wu = wg + static_cast<size_t>(a.ff) * K;
+    const bf16_t* x_row[RT];
+    float weight[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = rt * 16 + r;
+        const int pair = a.sorted[begin + min(row, rows - 1)];
+        x_row[rt] = x + static_cast<size_t>(pair / a.top) * K;
+        weight[rt] = row < rows ? a.pair_weight[pair] : 0.f;
+    }
+    floatx4 acc_g[RT], acc_u[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc_g[rt] = acc_u[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + g * 8;
+        const bool k_ok = k < K;
+        const uint4 zero = uint4{0, 0, 0, 0};
+        const uint4 bg = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wg + k) : zero;
+        const uint4 bu = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wu + k) : zero;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const uint4 raw = k_ok ? *reinterpret_cast<const uint4*>(x_row[rt] + k) : zero;
+            const bf16x8 af = scaled_fragment(raw, weight[rt]);
+            acc_g[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bg), acc_g[rt], 0, 0, 0);
+            acc_u[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bu), acc_u[rt], 0, 0, 0);
+        }
+    }
+    if (!col_ok) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = rt * 16 + g * 4 + i;
+            if (row < rows)
+                act[static_cast<size_t>(begin + row) * a.ff + c0 + r] =
+                    from_float<bf16_t>(clamped_glu(acc_g[rt][i], acc_u[rt][i], a.limit, a.alpha, a.offset));
+        }
+}
+
+template <int RT>
+__global__ void __launch_bounds__(256)
+experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ w_down, float* __restrict__ parts,
+                         ExpertArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= *a.n_tiles) return;
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int c0 = (blockIdx.y * 4 + wave) * 16;
+    if (c0 >= a.hidden) return;
+    const int expert = a.tile_expert[tile];
+    const int begin = a.tile_begin[tile];
+    const int rows = a.tile_count[tile];
+    const int K = a.ff;
+    const bool col_ok = c0 + r < a.hidden;
+    const bf16_t* wd = w_down + (static_cast<size_t>(expert) * a.hidden + min(c0 + r, a.hidden - 1)) * K;
+    floatx4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + g * 8;
+        const bool k_ok = k < K;
+        const uint4 zero = uint4{0, 0, 0, 0};
+        const uint4 b = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wd + k) : zero;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const int row = rt * 16 + r;
+            const uint4 raw = (k_ok && row < rows)
+                ? *reinterpret_cast<const uint4*>(act + static_cast<size_t>(begin + row) * K + k) : zero;
+            acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw),
+                                                              __builtin_bit_cast(bf16x8, b), acc[rt], 0, 0, 0);
+        }
+    }
+    if (!col_ok) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = rt * 16 + g * 4 + i;
+            if (row < rows) parts[static_cast<size_t>(a.sorted[begin + row]) * a.hidden + c0 + r] = acc[rt][i];
+        }
+}
+
+// The plain forms: tiles of up to 16 rows, 16 columns a workgroup, one thread per result.
+template <typename T>
+__global__ void __launch_bounds__(256)
+experts_gate_up_plain_kernel(const T* __restrict__ x, const T* __restrict__ w_gate_up, T* __restrict__ act, ExpertArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= *a.n_tiles) return;
+    const int row = threadIdx.x / 16;
+    const int col = blockIdx.y * 16 + threadIdx.x % 16;
+    if (row >= a.tile_count[tile] || col >= a.ff) return;
+    const int expert = a.tile_expert[tile];
+    const int place = a.tile_begin[tile] + row;
+    const int pair = a.sorted[place];
+    const float w = a.pair_weight[pair];
+    const int K = a.hidden;
+    const T* x_row = x + static_cast<size_t>(pair / a.top) * K;
+    const T* wg = w_gate_up + (static_cast<size_t>(expert) * 2 * a.ff + col) * K;
+    const T* wu = wg + static_cast<size_t>(a.ff) * K;
+    float sum_g = 0.f, sum_u = 0.f;
+    for (int k = 0; k < K; ++k) {
+        const float v = to_float(from_float<T>(to_float(x_row[k]) * w));  // the scaled input, as the storage type holds it
+        sum_g = fmaf(v, to_float(wg[k]), sum_g);
+        sum_u = fmaf(v, to_float(wu[k]), sum_u);
+    }
+    act[static_cast<size_t>(place) * a.ff + col] = from_float<T>(clamped_glu(sum_g, sum_u, a.limit, a.alpha, a.offset));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+experts_down_plain_kernel(const T* __restrict__ act, const T* __restrict__ w_down, float* __restrict__ parts, ExpertArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= *a.n_tiles) return;
+    const int row = threadIdx.x / 16;
+    const int col = blockIdx.y * 16 + threadIdx.x % 16;
+    if (row >= a.tile_count[tile] || col >= a.hidden) return;
+    const int expert = a.tile_expert[tile];
+    const int place = a.tile_begin[tile] + row;
+    const int K = a.ff;
+    const T* a_row = act + static_cast<size_t>(place) * K;
+    const T* wd = w_down + (static_cast<size_t>(expert) * a.hidden + col) * K;
+    float sum = 0.f;
+    for (int k = 0; k < K; ++k) sum = fmaf(to_float(a_row[k]), to_float(wd[k]), sum);
+    parts[static_cast<size_t>(a.sorted[place]) * a.hidden + col] = sum;
+}
+
+}  // namespace
+
+CIE_API int cie_experts_route(void* stream, const float* logits, int tokens, int experts, int top, int tile_rows,
+                              int* pair_expert, float* pair_weight, int* sorted, int* tile_expert, int* tile_begin,
+                              int* tile_count, int* n_tiles) {
+    if (tokens < 0 || experts < 1 || experts > kMaxExperts || top < 1 || top > experts || tile_rows < 1)
+        return CIE_BAD_ARGUMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (tokens > 0) {
+        route_kernel<<<(tokens + 3) / 4, 256, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight);
+        if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
+    }
+    arrange_kernel<<<1, 1024, 0, s>>>(pair_expert, tokens * top, experts, tile_rows, sorted, tile_expert, tile_begin,
+                                      tile_count, n_tiles);
+    return cie_after_launch();
+}
+
+// act [pairs, ff] in the storage type, rows in sorted order.  `mfma` != 0: the matrix-core form (bfloat16, hidden
+// and ff multiples of 8, tile_rows 16 * row_tiles with row_tiles 1, 2 or 4); else tile_rows must be <= 16.
+CIE_API int cie_experts_gate_up(void* stream, int dtype, int mfma, const void* x, const void* w_gate_up, void* act,
+                                const int* sorted, const float* pair_weight, const int* tile_expert,
+                                const int* tile_begin, const int* tile_count, const int* n_tiles, int max_tiles,
+                                int tile_rows, int top, int hidden, int ff, float limit, float alpha, float offset) {
+    if (max_tiles < 0 || top < 1 || hidden < 1 || ff < 1 || !(limit > 0.f) || tile_rows < 1) return CIE_BAD_ARGUMENT;
+    if (max_tiles == 0) return CIE_OK;
+    const ExpertArgs a{sorted, pair_weight, tile_expert, tile_begin, tile_count, n_tiles, top, hidden, ff, limit, alpha, offset};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (mfma) {
+        if (dtype != CIE_BF16 || hidden % 8 || ff % 8) return CIE_BAD_ARGUMENT;
+        dim3 grid(max_tiles, (ff + 63) / 64);
+        const bf16_t* xs = static_cast<const bf16_t*>(x);
+        const bf16_t* ws = static_cast<const bf16_t*>(w_gate_up);
+        bf16_t* as = static_cast<bf16_t*>(act);
+        if (tile_rows == 16) experts_gate_up_mfma_kernel<1><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        else if (tile_rows == 32) experts_gate_up_mfma_kernel<2><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        else if (tile_rows == 64) experts_gate_up_mfma_kernel<4><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        else return CIE_BAD_ARGUMENT;
+        return cie_after_launch();
+    }
+    if (tile_rows > 16) return CIE_BAD_ARGUMENT;
+    dim3 grid(max_tiles, (ff + 15) / 16);
+    if (dtype == CIE_F32)
+        experts_gate_up_plain_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), static_cast<const float*>(w_gate_up),
+                                                                static_cast<float*>(act), a);
+    else if (dtype == CIE_BF16)
+        experts_gate_up_plain_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_gate_up),
+                                                                 static_cast<bf16_t*>(act), a);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// parts [pairs, hidden] float32, row p the pair p = token * top + k.
+CIE_API int cie_experts_down(void* stream, int dtype, int mfma, const void* act, const void* w_down, float* parts,
+                             const int* sorted, const int* tile_expert, const int* tile_begin, const int* tile_count,
+                             const int* n_tiles, int max_tiles, int tile_rows, int top, int hidden, int ff) {
+    if (max_tiles < 0 || top < 1 || hidden < 1 || ff < 1 || tile_rows < 1) return CIE_BAD_ARGUMENT;
+    if (max_tiles == 0) return CIE_OK;
+    const ExpertArgs a{sorted, nullptr, tile_expert, tile_begin, tile_count, n_tiles, top, hidden, ff, 1.f, 1.f, 0.f};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (mfma) {
+        if (dtype != CIE_BF16 || hidden % 8 || ff % 8) return CIE_BAD_ARGUMENT;
+        dim3 grid(max_tiles, (hidden + 63) / 64);
+        const bf16_t* as = static_cast<const bf16_t*>(act);
+        const bf16_t* ws = static_cast<const bf16_t*>(w_down);
+        if (tile_rows == 16) experts_down_mfma_kernel<1><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        else if (tile_rows == 32) experts_down_mfma_kernel<2><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        else if (tile_rows == 64) experts_down_mfma_kernel<4><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        else return CIE_BAD_ARGUMENT;
+        return cie_after_launch();
+    }
+    if (tile_rows > 16) return CIE_BAD_ARGUMENT;
+    dim3 grid(max_tiles, (hidden + 15) / 16);
+    if (dtype == CIE_F32)
+        experts_down_plain_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(act), static_cast<const float*>(w_down), parts, a);
+    else if (dtype == CIE_BF16)
+        experts_down_plain_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(act), static_cast<const bf16_t*>(w_down), parts, a);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

@@ -96,10 +96,12 @@ def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype,
 
 # ---------------------------------------------------------------------------
 def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None,
-          feed: Optional[torch.Tensor] = None, pool: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``out[t] = float32(table[ids[t]])``; ids int32 [T] (already checked against the vocabulary).
+          feed: Optional[torch.Tensor] = None, pool: Optional[torch.Tensor] = None, scale: float = 1.0,
+          rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t] = float32(table[ids[t]]) * scale``; ids int32 [T] (already checked against the vocabulary).
     With ``feed`` (int32 [T]) and ``pool`` (int32): row t takes ``pool[feed[t]]`` as its id where
-    ``feed[t] >= 0`` (tokens another kernel left on the device; ``feed[t]`` must index ``pool``)."""
+    ``feed[t] >= 0`` (tokens another kernel left on the device; ``feed[t]`` must index ``pool``).
+    ``rows`` ([T, hidden] in the table's dtype) also takes the same values, rounded to that dtype."""
     _gpu("table", table, dims=2)
     _gpu("ids", ids, torch.int32, 1)
     vocab, hidden = table.shape
@@ -114,9 +116,13 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     _gpu("out", out, torch.float32, 2)
     if not (out.shape == (tokens, hidden)):
         raise ValueError(f"out must be {(tokens, hidden)}, is {tuple(out.shape)}")
+    if rows is not None:
+        _gpu("rows", rows, table.dtype, 2)
+        if not (rows.shape == (tokens, hidden)):
+            raise ValueError(f"rows must be {(tokens, hidden)}, is {tuple(rows.shape)}")
     _run("cie_embed", load_library().cie_embed(_stream(), _i(_code(table.dtype)), _ptr(table), _ptr(ids), _ptr(feed),
-                                               _ptr(pool if feed is not None else None), _ptr(out), _i(tokens),
-                                               _i(hidden), _i(vocab)))
+                                               _ptr(pool if feed is not None else None), _ptr(out), _ptr(rows),
+                                               _i(tokens), _i(hidden), _i(vocab), _f(scale)))
     return out
 
 
@@ -1064,3 +1070,286 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
         _i(block_width), _ptr(rate), _ptr(state), _ptr(past), _ptr(seq_slot), _ptr(q_start_loc), _ptr(out),
         _i(sequences), _i(channels), _i(taps), _i(segments)))
     return out
+
+
+# ---------------------------------------------------------------------------
+def branch_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                    out_dtype: torch.dtype, parts: Optional[torch.Tensor] = None,
+                    want_rows: bool = True) -> Optional[torch.Tensor]:
+    """``residual += y / sqrt(mean(y^2) + eps) * weight`` with ``y = branch + sum_p parts[:, p]``, row by row, in
+    float32 and in place.  ``branch`` [T, H] float32 or ``out_dtype`` (or ``None``), ``parts`` float32 [T, P, H]
+    (or ``None``), ``weight`` float32 [H] as it multiplies.  Returns the new stream rounded to ``out_dtype``
+    (``want_rows``), which is what the next sublayer's products read."""
+    _gpu("residual", residual, torch.float32, 2)
+    tokens, hidden = residual.shape
+    _gpu("weight", weight, torch.float32, 1)
+    if not (weight.shape[0] == hidden and hidden <= MAX_NORM_WIDTH and eps > 0):
+        raise ValueError(f"weight {tuple(weight.shape)}, hidden {hidden}, eps {eps} do not fit the norm kernel")
+    if branch is None and parts is None:
+        raise ValueError("nothing to add")
+    if branch is not None:
+        _gpu("branch", branch, dims=2)
+        if not (branch.shape == residual.shape and branch.dtype in (torch.float32, out_dtype)):
+            raise ValueError(f"branch {tuple(branch.shape)} {branch.dtype} does not fit {tuple(residual.shape)} {out_dtype}")
+    n_parts = 0
+    if parts is not None:
+        _gpu("parts", parts, torch.float32, 3)
+        if not (parts.shape[0] == tokens and parts.shape[2] == hidden):
+            raise ValueError(f"parts {tuple(parts.shape)} do not fit {tuple(residual.shape)}")
+        n_parts = parts.shape[1]
+    rows = torch.empty((tokens, hidden), dtype=out_dtype, device=residual.device) if want_rows else None
+    _run("cie_branch_norm_add", load_library().cie_branch_norm_add(
+        _stream(), _i(_code(branch.dtype if branch is not None else torch.float32)), _i(_code(out_dtype)),
+        _ptr(residual), _ptr(branch), _ptr(parts), _i(n_parts), _ptr(weight), _ptr(rows), _i(tokens), _i(hidden), _f(eps)))
+    return rows
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, offset: float) -> torch.Tensor:
+    """``g * sigmoid(alpha * g) * (u + offset)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)`` for
+    gate_up [T, 2I] (gate half first)."""
+    _gpu("gate_up", gate_up, dims=2)
+    tokens, twice = gate_up.shape
+    if twice % 2 or not limit > 0:
+        raise ValueError(f"gate_up rows must be even and the limit positive, got {twice}, {limit}")
+    out = torch.empty((tokens, twice // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _run("cie_clamped_glu", load_library().cie_clamped_glu(_stream(), _i(_code(gate_up.dtype)), _ptr(gate_up), _ptr(out),
+                                                           _i(tokens), _i(twice // 2), _f(limit), _f(alpha), _f(offset)))
+    return out
+
+
+def soft_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place on a float32 tensor."""
+    _gpu("x", x, torch.float32)
+    if not cap > 0:
+        raise ValueError(f"the cap must be positive, got {cap}")
+    _run("cie_soft_cap", load_library().cie_soft_cap(_stream(), _ptr(x), _i(x.numel()), _f(cap)))
+    return x
+
+
+# ---------------------------------------------------------------------------
+NORM_MODES = {None: 0, "unit": 1, "weight": 2}
+SCORED_MFMA_DIMS = ((64, 64), (128, 128), (64, 128), (128, 64))  # (key, value) head sizes of the matrix-core form
+
+
+def _check_kv_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype, kv_heads: int, dim: int,
+                    vdim: int) -> int:
+    _gpu("k_pool", k_pool, dtype, 4)
+    _gpu("v_pool", v_pool, dtype, 4)
+    pages, heads, page_size, width = k_pool.shape
+    if not (heads == kv_heads and width == dim and tuple(v_pool.shape) == (pages, kv_heads, vdim, page_size)):
+        raise ValueError(f"pools {tuple(k_pool.shape)}, {tuple(v_pool.shape)} do not fit {kv_heads} heads of {dim} and {vdim}")
+    return page_size
+
+
+def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: int, kv_heads: int, dim: int, vdim: int,
+                  kernel_dim: int, kernel_vdim: int, norm: Optional[str], q_weight: Optional[torch.Tensor],
+                  k_weight: Optional[torch.Tensor], eps: float, temperature: Optional[tuple[float, int]],
+                  positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
+                  block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, tokens: int,
+                  write_kv: bool = True) -> torch.Tensor:
+    """From projected rows ``proj`` [T, >= ...] (queries at column ``offsets[0]``, keys at ``offsets[1]``, values at
+    ``offsets[2]``, heads of ``dim`` / ``dim`` / ``vdim`` numbers) to queries ``[T, q_heads * kernel_dim]`` and the
+    token's cache entries: per-head RMS norm of queries and keys (``norm``: ``None``, ``"unit"`` or ``"weight"`` with
+    float32 weights [dim]), the queries times ``1 + coef * ln(floor((p + 1) / every) + 1)`` (``temperature = (coef,
+    every)``), heads zero-padded up to the kernels' sizes."""
+    if not (proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1):
+        raise ValueError("proj must be 2-d on the GPU with unit inner stride")
+    dtype = proj.dtype
+    q_off, k_off, v_off = offsets
+    need = max(q_off + q_heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim)
+    if not (proj.shape[0] >= tokens and proj.shape[1] >= need and min(offsets) >= 0):
+        raise ValueError(f"proj {tuple(proj.shape)} too small for {tokens} tokens of {need} numbers")
+    if norm not in NORM_MODES:
+        raise ValueError(f"norm must be one of {list(NORM_MODES)}, got {norm!r}")
+    if norm == "weight":
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            if w is None:
+                raise ValueError(f"{name} is missing")
+            _gpu(name, w, torch.float32, 1)
+            if w.shape[0] != dim:
+                raise ValueError(f"{name} must be [{dim}], is {tuple(w.shape)}")
+    if kernel_dim < dim or kernel_vdim < vdim:
+        raise ValueError("the kernels' head sizes must hold the projection's")
+    page_size = _check_kv_pools(k_pool, v_pool, dtype, kv_heads, kernel_dim, kernel_vdim)
+    _gpu("block_table", block_table, torch.int32, 2)
+    for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(name, meta, torch.int32, 1)
+        if not (meta.shape[0] >= tokens):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+    _gpu("seq_slot", seq_slot, torch.int32, 1)
+    coef, every = temperature if temperature else (0.0, 0)
+    if temperature and every < 1:
+        raise ValueError("the temperature's period must be positive")
+    q_out = torch.empty((tokens, q_heads * kernel_dim), dtype=dtype, device=proj.device)
+    _run("cie_heads_prepare", load_library().cie_heads_prepare(
+        _stream(), _i(_code(dtype)), _ptr(proj), _i(proj.stride(0)), _i(q_off), _i(k_off), _i(v_off), _ptr(q_weight),
+        _ptr(k_weight), _i(NORM_MODES[norm]), _f(eps), _f(coef), _i(every), _ptr(positions), _ptr(seq_of_token),
+        _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(q_out), _ptr(k_pool), _ptr(v_pool),
+        _i(tokens), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(kernel_dim), _i(kernel_vdim), _i(page_size),
+        _i(1 if write_kv else 0)))
+    return q_out
+
+
+def _check_score_shape(q_heads: int, slopes, sinks, softcap) -> None:
+    for name, t in (("slopes", slopes), ("sinks", sinks)):
+        if t is not None:
+            _gpu(name, t, torch.float32, 1)
+            if t.shape[0] != q_heads:
+                raise ValueError(f"{name} must be [{q_heads}], is {tuple(t.shape)}")
+    if softcap is not None and not softcap > 0:
+        raise ValueError(f"the cap on the scores must be positive, got {softcap}")
+
+
+def _check_gate(gate, tokens: int, q_heads: int, dtype: torch.dtype) -> int:
+    if gate is None:
+        return 0
+    if not (gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == dtype
+            and gate.shape[0] >= tokens and gate.shape[1] >= q_heads):
+        raise ValueError(f"gate {tuple(gate.shape)} {gate.dtype} does not hold {tokens} rows of {q_heads} heads")
+    return gate.stride(0)
+
+
+def scored_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, block_table: torch.Tensor,
+                             positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor, tokens: int,
+                             q_heads: int, kv_heads: int, dim: int, vdim: int, window: Optional[int], scale: float,
+                             softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
+                             sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of each token over its request's cached keys with shaped scores (see ``csrc/attention_scored.hip``):
+    ``q`` [T, q_heads * dim]; returns [T, q_heads * vdim].  ``gate`` [T, >= q_heads] (a view is fine): head h's output
+    is multiplied by ``sigmoid(gate[t, h])``.  float32 or bfloat16."""
+    _gpu("q", q, dims=2)
+    if not (q.shape == (tokens, q_heads * dim) and q_heads % kv_heads == 0 and dim % 8 == 0 and vdim % 8 == 0
+            and dim <= 256 and vdim <= 256):
+        raise ValueError(f"q {tuple(q.shape)} does not fit {tokens} tokens of {q_heads} heads of {dim} (multiples of 8 up to 256)")
+    page_size = _check_kv_pools(k_pool, v_pool, q.dtype, kv_heads, dim, vdim)
+    _gpu("block_table", block_table, torch.int32, 2)
+    for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(name, meta, torch.int32, 1)
+        if not (meta.shape[0] >= tokens):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+    _gpu("seq_slot", seq_slot, torch.int32, 1)
+    _check_score_shape(q_heads, slopes, sinks, softcap)
+    gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
+    out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
+    _run("cie_scored_attention_generic", load_library().cie_scored_attention_generic(
+        _stream(), _i(_code(q.dtype)), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _i(block_table.shape[1]),
+        _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(gate), _i(gate_stride), _ptr(out), _i(tokens),
+        _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(window or 0), _f(scale), _f(softcap or 0.0),
+        _ptr(slopes), _ptr(sinks)))
+    return out
+
+
+def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, block_table: torch.Tensor,
+                          tile_seq: Optional[torch.Tensor], tile_q0: Optional[torch.Tensor], n_tiles: int,
+                          seq_slot: torch.Tensor, seq_start: torch.Tensor, seq_q_len: torch.Tensor,
+                          q_start_loc: torch.Tensor, tokens: int, q_heads: int, kv_heads: int, dim: int, vdim: int,
+                          tokens_per_tile: int, row_tiles: int, window: Optional[int], scale: float,
+                          softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
+                          sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same on the matrix cores (bfloat16, (dim, vdim) in ``SCORED_MFMA_DIMS``, pages of a power of two >= 4):
+    tiles of ``tokens_per_tile`` consecutive tokens of one sequence (``tile_seq``, ``tile_q0`` int32 [n_tiles]; both
+    ``None``: tile i is sequence i's first), whose rows times the heads per key head fill ``row_tiles`` tiles of 16."""
+    _gpu("q", q, torch.bfloat16, 2)
+    if not (q.shape == (tokens, q_heads * dim) and q_heads % kv_heads == 0 and (dim, vdim) in SCORED_MFMA_DIMS):
+        raise ValueError(f"q {tuple(q.shape)} / heads of {dim}, {vdim} are not what the matrix-core form takes")
+    page_size = _check_kv_pools(k_pool, v_pool, q.dtype, kv_heads, dim, vdim)
+    if page_size < 4 or page_size & (page_size - 1):
+        raise ValueError(f"pages must hold a power of two >= 4 keys, hold {page_size}")
+    group = q_heads // kv_heads
+    if row_tiles not in (1, 2, 4) or tokens_per_tile < 1 or tokens_per_tile * group > 16 * row_tiles:
+        raise ValueError(f"{tokens_per_tile} tokens of {group} heads do not fit {row_tiles} tiles of 16 rows")
+    _gpu("block_table", block_table, torch.int32, 2)
+    if (tile_seq is None) != (tile_q0 is None):
+        raise ValueError("tile_seq and tile_q0 come together")
+    if tile_seq is not None:
+        for name, t in (("tile_seq", tile_seq), ("tile_q0", tile_q0)):
+            _gpu(name, t, torch.int32, 1)
+            if t.shape[0] < n_tiles:
+                raise ValueError(f"{name} has {t.shape[0]} entries for {n_tiles} tiles")
+    sequences = seq_slot.shape[0]
+    for name, meta, least in (("seq_slot", seq_slot, 1), ("seq_start", seq_start, sequences),
+                              ("seq_q_len", seq_q_len, sequences), ("q_start_loc", q_start_loc, sequences)):
+        _gpu(name, meta, torch.int32, 1)
+        if meta.shape[0] < least:
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
+    if tile_seq is None and n_tiles > sequences:
+        raise ValueError(f"{n_tiles} tiles for {sequences} sequences")
+    _check_score_shape(q_heads, slopes, sinks, softcap)
+    gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
+    out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
+    _run("cie_scored_attention_mfma", load_library().cie_scored_attention_mfma(
+        _stream(), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _i(block_table.shape[1]), _ptr(tile_seq),
+        _ptr(tile_q0), _i(n_tiles), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len), _ptr(q_start_loc), _ptr(gate),
+        _i(gate_stride), _ptr(out), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(tokens_per_tile),
+        _i(row_tiles), _i(window or 0), _f(scale), _f(softcap or 0.0), _ptr(slopes), _ptr(sinks)))
+    return out
+
+
+# ---------------------------------------------------------------------------
+MAX_EXPERTS = 1024
+EXPERT_TILE_ROWS = (16, 32, 64)  # rows of one expert that a workgroup of the matrix-core forms takes
+
+
+class ExpertRoute:
+    """What ``experts_route`` leaves on the device for the expert products of one step."""
+
+    __slots__ = ("pair_expert", "pair_weight", "sorted", "tile_expert", "tile_begin", "tile_count", "n_tiles",
+                 "max_tiles", "tile_rows", "top", "pairs")
+
+
+def experts_route(logits: torch.Tensor, top: int, tile_rows: int = 16) -> ExpertRoute:
+    """Scores ``sigmoid(logits)`` (float32 [T, E]), the ``top`` largest per token (lowest index first among equals),
+    and the (token, choice) pairs sorted by expert in tiles of at most ``tile_rows`` rows.  Nothing comes back to
+    the host: grids are sized for ``max_tiles`` and the kernels read the true count."""
+    _gpu("logits", logits, torch.float32, 2)
+    tokens, experts = logits.shape
+    if not (1 <= top <= experts <= MAX_EXPERTS and tile_rows >= 1):
+        raise ValueError(f"{top} of {experts} experts (at most {MAX_EXPERTS}) in tiles of {tile_rows}")
+    route = ExpertRoute()
+    pairs = tokens * top
+    route.pairs, route.top, route.tile_rows = pairs, top, tile_rows
+    route.max_tiles = min(pairs, pairs // tile_rows + experts)
+    ints = torch.empty(2 * pairs + 3 * max(route.max_tiles, 1) + 1, dtype=torch.int32, device=logits.device)
+    route.pair_expert, route.sorted = ints[:pairs], ints[pairs: 2 * pairs]
+    base = 2 * pairs
+    width = max(route.max_tiles, 1)
+    route.tile_expert, route.tile_begin, route.tile_count = (ints[base + i * width: base + (i + 1) * width] for i in range(3))
+    route.n_tiles = ints[base + 3 * width:]
+    route.pair_weight = torch.empty(pairs, dtype=torch.float32, device=logits.device)
+    _run("cie_experts_route", load_library().cie_experts_route(
+        _stream(), _ptr(logits), _i(tokens), _i(experts), _i(top), _i(tile_rows), _ptr(route.pair_expert),
+        _ptr(route.pair_weight), _ptr(route.sorted), _ptr(route.tile_expert), _ptr(route.tile_begin),
+        _ptr(route.tile_count), _ptr(route.n_tiles)))
+    return route
+
+
+def experts_forward(x: torch.Tensor, route: ExpertRoute, w_gate_up: torch.Tensor, w_down: torch.Tensor, limit: float,
+                    alpha: float, offset: float, mfma: bool) -> torch.Tensor:
+    """The chosen experts' outputs, float32 ``[T, top, hidden]``: row (t, k) is expert ``k`` of token t run on
+    ``weight * x[t]``.  ``w_gate_up`` [E, 2 * ff, hidden] (gate rows first), ``w_down`` [E, hidden, ff]."""
+    _gpu("x", x, dims=2)
+    tokens, hidden = x.shape
+    _gpu("w_gate_up", w_gate_up, x.dtype, 3)
+    _gpu("w_down", w_down, x.dtype, 3)
+    experts, twice, _ = w_gate_up.shape
+    ff = twice // 2
+    if not (w_gate_up.shape == (experts, 2 * ff, hidden) and w_down.shape == (experts, hidden, ff)
+            and tokens * route.top == route.pairs):
+        raise ValueError(f"expert weights {tuple(w_gate_up.shape)}, {tuple(w_down.shape)} do not fit rows {tuple(x.shape)}")
+    if mfma and not (x.dtype == torch.bfloat16 and hidden % 8 == 0 and ff % 8 == 0 and route.tile_rows in EXPERT_TILE_ROWS):
+        raise ValueError("the matrix-core form takes bfloat16, widths that are multiples of 8 and tiles of 16, 32 or 64 rows")
+    if not mfma and route.tile_rows > 16:
+        raise ValueError("the plain form takes tiles of up to 16 rows")
+    act = torch.empty((route.pairs, ff), dtype=x.dtype, device=x.device)
+    parts = torch.empty((tokens, route.top, hidden), dtype=torch.float32, device=x.device)
+    lib = load_library()
+    _run("cie_experts_gate_up", lib.cie_experts_gate_up(
+        _stream(), _i(_code(x.dtype)), _i(1 if mfma else 0), _ptr(x), _ptr(w_gate_up), _ptr(act), _ptr(route.sorted),
+        _ptr(route.pair_weight), _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count),
+        _ptr(route.n_tiles), _i(route.max_tiles), _i(route.tile_rows), _i(route.top), _i(hidden), _i(ff), _f(limit),
+        _f(alpha), _f(offset)))
+    _run("cie_experts_down", lib.cie_experts_down(
+        _stream(), _i(_code(x.dtype)), _i(1 if mfma else 0), _ptr(act), _ptr(w_down), _ptr(parts), _ptr(route.sorted),
+        _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count), _ptr(route.n_tiles),
+        _i(route.max_tiles), _i(route.tile_rows), _i(route.top), _i(hidden), _i(ff)))
+    return parts

@@ -1,4 +1,5 @@
-from . import attention, block, feed_forward, latent_attention, norm, position, recurrent  # noqa: F401  (fill the registries)
+from . import (attention, block, feed_forward, latent_attention, norm, position, recurrent,  # noqa: F401
+               routed_experts, scored_attention)  # (fill the registries)
 from .base import (
     BLOCKS,
     FEED_FORWARDS,

@@ -8,6 +8,9 @@ that can add its output into the residual itself (the fused decode products do)
 returns a ``RowSumsq`` or an ``Added`` instead, and the next norm then runs its
 cheaper form or rides along with the product behind it (``parts/linear.py``).
 
+``BranchNormBlock``: the sublayers read the stream itself and their outputs are normed before they are added:
+``h += norm1(mixer(h)); h += norm2(feed_forward(h))``.
+
 ``ParallelDepthBlock``: both branches read the same stream, and the next layer reads a weighted average of what
 the embedding and all layers so far left (below).
 """
@@ -23,7 +26,7 @@ from ..config.specs import LayerSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
-from .linear import Added, RawRows, RowSumsq
+from .linear import Added, RawRows, RowSumsq, StreamRows
 
 
 class PreNormBlock:
@@ -92,6 +95,53 @@ def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, rows=No
 
 
 register_part("block", "pre_norm", PreNormBlock)
+
+
+class BranchNormBlock(PreNormBlock):
+    """``h += norm1(mixer(h)); h += norm2(feed_forward(h))``: no norm in front of a sublayer, one on its output.
+    The stream is float32; each add (one kernel with the norm) also leaves the stream rounded to the activation
+    type, which the next sublayer's products read (in a float32 engine they read the stream itself).  A layer
+    without feed-forward has no second norm; a checkpoint that holds one all the same is accepted.  The norms are
+    of a kind with ``add_normed`` (``rms_norm_one_plus``)."""
+
+    reads_stream = True
+
+    def __init__(self, spec: LayerSpec) -> None:
+        super().__init__(spec)
+        self.has_feed_forward = spec.feed_forward.kind != "none"
+        for norm in (self.norm1, self.norm2):
+            if not hasattr(norm, "add_normed"):
+                raise ValueError("this arrangement takes norms that can add a normed branch (rms_norm_one_plus)")
+
+    def _parts(self):
+        parts = [("norm1", self.norm1), ("mixer", self.mixer)]
+        if self.has_feed_forward:
+            parts += [("norm2", self.norm2), ("feed_forward", self.feed_forward)]
+        return parts
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        out = super().expected_tensors(prefix)
+        if not self.has_feed_forward:
+            for name, spec in self.norm2.expected_tensors(f"{prefix}{self.spec.name_of('norm2')}.").items():
+                out[name] = replace(spec, optional=True)
+        return out
+
+    def forward(self, residual: torch.Tensor, pending, batch, view, writes: bool = True):
+        if isinstance(pending, StreamRows) and pending.rows is not None:
+            x = pending.rows
+        elif pending is None or isinstance(pending, Added):
+            x = residual if self.dtype == torch.float32 else residual.to(self.dtype)
+        else:
+            raise ValueError("a branch that is still to be added cannot be handed to this arrangement")
+        mixed = self.mixer.forward(x, batch, view, writes)
+        x = self.norm1.add_normed(residual, mixed, self.dtype, want_rows=self.dtype != torch.float32)
+        if self.has_feed_forward:
+            fed = self.feed_forward.forward(residual if x is None else x)
+            x = self.norm2.add_normed(residual, fed, self.dtype, want_rows=self.dtype != torch.float32)
+        return residual, StreamRows(x)
+
+
+register_part("block", "branch_norm", BranchNormBlock)
 
 
 @dataclass

@@ -136,6 +136,23 @@ class Added:
 
 
 @dataclass
+class StreamRows(Added):
+    """An ``Added`` that also carries the whole stream rounded to the activation type (``rows``): what a layer
+    whose sublayers read the stream itself, not a norm of it, hands to the next one."""
+
+    rows: Optional[torch.Tensor] = None
+
+
+@dataclass
+class SummedBranch:
+    """A branch output that is still a sum: ``main`` [T, H] (or ``None``) plus the ``P`` rows of each token in
+    ``parts`` (float32 [T, P, H]).  Whoever adds the branch sums them, in that order."""
+
+    main: Optional[torch.Tensor]
+    parts: Optional[torch.Tensor]
+
+
+@dataclass
 class RawRows:
     """Stands where an RMSNorm's output would, before anything was computed: the rows are the norm ``norm``
     of the float32 stream ``residual``.  Only a mixer that says ``takes_raw_rows`` is shown it (the attention

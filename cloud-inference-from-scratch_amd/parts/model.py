@@ -16,7 +16,7 @@ from ..weights.loader import torch_dtype
 from ..weights.tensors import TensorSpec
 from .base import BLOCKS, build_part
 from .block import normalise
-from .linear import linear
+from .linear import StreamRows, linear
 
 
 def _blocks(spec: ModelSpec) -> list[Any]:
@@ -128,9 +128,16 @@ class DecoderModel:
         if self.keeps_history:
             history = torch.empty((len(self.spec.order) + 1, batch.token_ids.shape[0], self.embedding.shape[1]),
                                   dtype=torch.float32, device=self.embedding.device)
+        first = self.blocks[self.spec.order[0].layer] if self.spec.order else None
+        rows = None
+        if getattr(first, "reads_stream", False) and self.embedding.dtype != torch.float32:
+            # a first layer whose products read the stream itself: the embedding kernel also leaves it in their type
+            rows = torch.empty((batch.token_ids.shape[0], self.embedding.shape[1]), dtype=self.embedding.dtype,
+                               device=self.embedding.device)
         residual = ops.embed(self.embedding, batch.token_ids, feed=batch.token_feed, pool=batch.token_pool,
-                             out=history[0] if history is not None else None)
-        pending = None
+                             out=history[0] if history is not None else None, scale=self.spec.embedding_scale,
+                             rows=rows)
+        pending = StreamRows(rows) if rows is not None else None
         for call in self.spec.order:
             block = self.blocks[call.layer]
             extra = {"history": history} if getattr(block, "keeps_history", False) else {}
@@ -138,4 +145,7 @@ class DecoderModel:
         if batch.logit_rows.shape[0] == 0:  # a step of prompt portions that end before their prompts do
             return torch.empty((0, self.head.shape[0]), dtype=torch.float32, device=residual.device)
         selected = normalise(self.final_norm, residual, pending, self.dtype, rows=batch.logit_rows)
-        return linear(selected, self.head, None, out_dtype=torch.float32)
+        logits = linear(selected, self.head, None, out_dtype=torch.float32)
+        if self.spec.logit_softcap is not None:
+            ops.soft_cap_(logits, self.spec.logit_softcap)
+        return logits

@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
-from .linear import Added, RowSumsq, ScaledRows
+from .linear import Added, RowSumsq, ScaledRows, SummedBranch
 
 
 class RMSNorm(Part):
@@ -89,5 +89,29 @@ class ScalarRMSNorm(Part):
         return ops.add_rmsnorm(residual, branch, self.weight_f32, self.eps, out_dtype, rows=rows)
 
 
+class OnePlusRMSNorm(RMSNorm):
+    """RMS norm whose checkpoint weight lies around zero: ``x * rsqrt(mean(x^2) + eps) * (1 + w)``.  The sum
+    ``1 + w`` is made once, in float32, when the weight is bound, and the tensor is named like the norm itself
+    (no ``.weight``).  ``add_normed`` is the form a layer uses that norms its branches' outputs:
+    ``residual += norm(branch)``."""
+
+    folds_into_products = False  # (the products' norm epilogues multiply by a weight in the activation type)
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {prefix.rstrip("."): TensorSpec((self.size,), init="normal", keeps_float32=True)}
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        Part.bind(self, tensors, prefix, dtype, device)
+        self.weight = (1.0 + tensors[prefix.rstrip(".")].float()).contiguous()
+        self.weight_f32 = self.weight
+
+    def add_normed(self, residual: torch.Tensor, branch, out_dtype: torch.dtype, want_rows: bool = True):
+        """``residual += norm(branch)`` in float32; returns the new stream in ``out_dtype`` (if wanted).
+        ``branch`` is a tensor or a ``SummedBranch``."""
+        main, parts = (branch.main, branch.parts) if isinstance(branch, SummedBranch) else (branch, None)
+        return ops.branch_norm_add(residual, main, self.weight, self.eps, out_dtype, parts=parts, want_rows=want_rows)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "rms_norm_one_plus", OnePlusRMSNorm)
 register_part("norm", "rms_norm_scalar", ScalarRMSNorm)

@@ -1,0 +1,187 @@
+"""Grouped-query softmax attention over a window of the paged cache, without rotation, whose scores are shaped by
+the position in other ways.  Every step is a parameter of the part and may be left out:
+
+* a per-head RMS norm of queries and keys (``qk_norm``: ``"weight"`` with one weight vector for all query heads
+  and one for all key heads, ``"unit"`` without weights, ``None``);
+* a factor on the queries that grows with the logarithm of the position (``q_temperature = (coef, every)``:
+  ``1 + coef * ln(floor((p + 1) / every) + 1)``);
+* ``score = q . k * scale``, then a smooth cap (``softcap``: ``c * tanh(score / c)``), then a bias on the distance
+  itself (``slope_base = b``: head h of H loses ``2^(-b (h + 1) / H) * (i - j)``);
+* a window (``window``: the token itself and the ``window - 1`` before it);
+* a sink (``sink``: one learned number per head whose exponential stands in the softmax's denominator, and
+  nowhere else);
+* a gate on every head's output (``head_gate``: ``sigmoid(W_g x)_h``, read from the layer's own input);
+* key and value heads of different sizes.
+
+One product makes queries, keys, values and gate logits; one kernel norms and scales the heads, lays the queries
+out and writes the cache (``ops.heads_prepare``); the attention kernel shapes the scores, and applies sink and
+gate in its epilogue: bfloat16 with head sizes up to 128 on the matrix cores (``ops.scored_attention_mfma``, the
+heads zero-padded to 64 or 128 numbers: no score and no output changes), anything else, and float32, in the
+generic form.  Norm statistics, the logarithm, scores, softmax, value sums and the gate are float32.
+"""
+
+from __future__ import annotations
+
+import warnings
+from typing import Optional
+
+import torch
+
+from ..cache.manager import PagedKV
+from ..kernels import ops
+from ..weights.tensors import TensorSpec
+from .base import Part, register_part
+from .linear import linear
+
+_SAID_GENERIC: set = set()
+
+
+def _round8(n: int) -> int:
+    return -(-n // 8) * 8
+
+
+class ScoredAttention(Part):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                 scale: float, eps: float, window: Optional[int] = None, qk_norm: Optional[str] = None,
+                 q_temperature: Optional[tuple] = None, softcap: Optional[float] = None,
+                 slope_base: Optional[float] = None, sink: bool = False, head_gate: bool = False) -> None:
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads),
+                            ("head_dim", head_dim), ("value_dim", value_dim)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer, got {value!r}")
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} key heads")
+        if max(head_dim, value_dim) > 256:
+            raise ValueError(f"heads of up to 256 numbers, got {head_dim} and {value_dim}")
+        if window is not None and window < 1:
+            raise ValueError("window must be positive")
+        if qk_norm not in ops.NORM_MODES:
+            raise ValueError(f"qk_norm must be one of {list(ops.NORM_MODES)}, got {qk_norm!r}")
+        if not eps > 0:
+            raise ValueError("eps must be positive")
+        if softcap is not None and not softcap > 0:
+            raise ValueError("softcap must be positive")
+        if q_temperature is not None:
+            coef, every = q_temperature
+            if isinstance(every, bool) or int(every) != every or every < 1:
+                raise ValueError(f"the temperature's period must be a positive integer, got {every!r}")
+            q_temperature = (float(coef), int(every))
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim = head_dim, value_dim
+        self.scale, self.eps, self.window = float(scale), float(eps), window
+        self.qk_norm, self.q_temperature, self.softcap = qk_norm, q_temperature, softcap
+        self.slope_base, self.sink, self.head_gate = slope_base, bool(sink), bool(head_gate)
+        # the head sizes the kernels and the cache see: those of the matrix-core form where it has them
+        sizes = tuple(next((s for s in (64, 128) if s >= n), None) for n in (head_dim, value_dim))
+        self.mfma_dims = sizes if sizes in ops.SCORED_MFMA_DIMS else None
+        self.kernel_dim, self.kernel_vdim = self.mfma_dims or (_round8(head_dim), _round8(value_dim))
+
+    def cache_need(self) -> PagedKV:
+        return PagedKV(self.num_kv_heads, self.kernel_dim, self.window,
+                       value_dim=self.kernel_vdim if self.kernel_vdim != self.kernel_dim else None)
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, g, d, v, width = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.hidden_size
+        out = {
+            prefix + "q": TensorSpec((h * d, width)),
+            prefix + "k": TensorSpec((g * d, width)),
+            prefix + "v": TensorSpec((g * v, width)),
+            prefix + "o": TensorSpec((width, h * v)),
+        }
+        if self.qk_norm == "weight":
+            out[prefix + "q.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
+            out[prefix + "k.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
+        if self.sink:
+            out[prefix + "sink"] = TensorSpec((h,), keeps_float32=True)
+        if self.head_gate:
+            out[prefix + "g"] = TensorSpec((h, width))
+        return out
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        h, g, d, v = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        blocks = [tensors[prefix + "q"], tensors[prefix + "k"], tensors[prefix + "v"]]
+        self.offsets = (0, h * d, h * d + g * d)
+        self.gate_offset = None
+        if self.head_gate:
+            # gate logits ride in the same product, on columns that start at a multiple of 8 (and the row is
+            # padded to one), so that the rows of the result stay 16-byte aligned
+            pad = lambda rows: blocks[0].new_zeros((rows, self.hidden_size))
+            used = h * d + g * d + g * v
+            if used % 8:
+                blocks.append(pad(8 - used % 8))
+            self.gate_offset = _round8(used)
+            blocks.append(tensors[prefix + "g"])
+            if h % 8:
+                blocks.append(pad(8 - h % 8))
+        self.w_in = torch.cat(blocks, dim=0).contiguous()
+        self.q_weight = self.k_weight = None
+        if self.qk_norm == "weight":
+            self.q_weight = tensors[prefix + "q.norm"].float().contiguous()
+            self.k_weight = tensors[prefix + "k.norm"].float().contiguous()
+        self.sinks = tensors[prefix + "sink"].float().contiguous() if self.sink else None
+        self.slopes = None
+        if self.slope_base is not None:
+            self.slopes = torch.tensor([2.0 ** (-self.slope_base * (i + 1) / h) for i in range(h)],
+                                       dtype=torch.float32, device=device)
+        w_o = tensors[prefix + "o"]
+        if self.kernel_vdim != v:  # the attention's rows hold padded heads: zero columns under the padding
+            wide = w_o.new_zeros((self.hidden_size, h, self.kernel_vdim))
+            wide[:, :, :v] = w_o.reshape(self.hidden_size, h, v)
+            w_o = wide.reshape(self.hidden_size, h * self.kernel_vdim)
+        self.w_o = w_o.contiguous()
+
+    def warm_up(self, rows: int) -> None:
+        blank = lambda width: torch.zeros((rows, width), dtype=self.w_in.dtype, device=self.w_in.device)
+        linear(blank(self.hidden_size), self.w_in)
+        linear(blank(self.num_heads * self.kernel_vdim), self.w_o)
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        proj = linear(x, self.w_in)
+        q = ops.heads_prepare(proj, self.offsets, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
+                              self.kernel_dim, self.kernel_vdim, self.qk_norm, self.q_weight, self.k_weight, self.eps,
+                              self.q_temperature, batch.positions, batch.seq_of_token, batch.seq_slot,
+                              view.block_table, view.k_pool, view.v_pool, batch.tokens, write_kv=writes)
+        gate = proj[:, self.gate_offset:] if self.head_gate else None
+        context = self.attend(q, gate, batch, view)
+        return linear(context, self.w_o)
+
+    def attend(self, q: torch.Tensor, gate, batch, view) -> torch.Tensor:
+        shape = dict(window=self.window, scale=self.scale, softcap=self.softcap, slopes=self.slopes,
+                     sinks=self.sinks, gate=gate)
+        h, g = self.num_heads, self.num_kv_heads
+        group = h // g
+        page_size = view.page_size
+        if q.dtype == torch.bfloat16 and self.mfma_dims and group <= 64 and page_size >= 4 and not page_size & (page_size - 1):
+            # rows of a tile: a token's heads of one key head, and as many tokens as fill the tile
+            least = 1 if group <= 16 else 2 if group <= 32 else 4
+            if batch.static_plan is not None and batch.static_plan.decode_rows in (None, batch.sequences):
+                # a captured step of single tokens: tile i is sequence i, nothing comes from the host
+                return ops.scored_attention_mfma(q, view.k_pool, view.v_pool, view.block_table, None, None,
+                                                 batch.sequences, batch.seq_slot, batch.seq_start, batch.seq_q_len,
+                                                 batch.q_start_loc, batch.tokens, h, g, self.kernel_dim,
+                                                 self.kernel_vdim, 1, least, **shape)
+            most = 4 if max(self.mfma_dims) <= 64 else 2
+            row_tiles = max(least, most if batch.max_q_len * group > 16 else 1)
+            while row_tiles > least and -(-batch.tokens * group // (16 * row_tiles)) * g < ops.compute_units():
+                row_tiles //= 2  # (fewer rows a tile where the tiles would not fill the compute units)
+            per_tile = (16 * row_tiles) // group
+            tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=None)
+            return ops.scored_attention_mfma(q, view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0, n_tiles,
+                                             batch.seq_slot, batch.seq_start, batch.seq_q_len, batch.q_start_loc,
+                                             batch.tokens, h, g, self.kernel_dim, self.kernel_vdim, per_tile,
+                                             row_tiles, **shape)
+        if q.dtype == torch.bfloat16 and (self.kernel_dim, self.kernel_vdim, group, page_size) not in _SAID_GENERIC:
+            _SAID_GENERIC.add((self.kernel_dim, self.kernel_vdim, group, page_size))
+            warnings.warn(f"bfloat16 attention with heads of {self.head_dim} and {self.value_dim} numbers, {group} query "
+                          f"heads per key head and pages of {page_size} takes the generic kernel (the matrix-core form "
+                          f"takes heads of up to 128 numbers, up to 64 heads per key head and pages of a power of two >= 4)",
+                          RuntimeWarning, stacklevel=2)
+        return ops.scored_attention_generic(q, view.k_pool, view.v_pool, view.block_table, batch.positions,
+                                            batch.seq_of_token, batch.seq_slot, batch.tokens, h, g, self.kernel_dim,
+                                            self.kernel_vdim, **shape)
+
+
+register_part("mixer", "scored_attention", ScoredAttention)
