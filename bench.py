@@ -5,7 +5,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
                     [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 32768]
                     [--mixed-portions 16,64,248] [--other-shapes 7b,14b]
-    python bench.py --design polosun [--design-shapes 3b,7b] [--design-layers 12]
+    python bench.py --design polosun|givizen [--design-shapes 3b,7b] [--design-layers 12]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -36,7 +36,10 @@ of equal width, feed-forward size, vocabulary and layer count, both with
 ``--design-layers`` layers and random weights: prefill of ``--prefill-tokens``
 tokens and decode at batch 1, ``--batch`` and 64 behind ``--context`` tokens,
 each with its share of the roofline of its own bytes and flops.  It prints one
-JSON line of its own.
+JSON line of its own.  ``--design givizen`` does the same for the Givizen design
+(window attention with shaped scores of two kinds in turn, each layer with
+routed experts and a shared one whose active sizes add up to the Qwen2.5
+shape's feed-forward).
 """
 
 from __future__ import annotations
@@ -274,11 +277,63 @@ def polosun_costs(config, batch: int, context: float, tokens: int, elem: int) ->
     return moved, 2.0 * tokens * (weights - head) + 2.0 * head + attention
 
 
+GIVIZEN_EXPERTS, GIVIZEN_TOP = 32, 4
+GIVIZEN_WINDOWS = (1024, 4096)
+
+
+def givizen_raw(shape: dict, layers: int) -> dict:
+    """A Givizen configuration with the width, vocabulary, head counts and head size of a Qwen2.5 shape: layers of
+    the two attention kinds in turn (windows of 1,024 and 4,096 tokens), each with 32 experts of which a token uses
+    4, and a shared expert; the four experts and the shared one together are as large as the shape's feed-forward."""
+    width = shape["hidden_size"]
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    dim = width // heads
+    expert_ff = shape["intermediate_size"] // (2 * GIVIZEN_TOP) // 64 * 64
+    shared_ff = shape["intermediate_size"] - GIVIZEN_TOP * expert_ff
+    mlp = {"kind": "moe", "router": {"experts": GIVIZEN_EXPERTS, "top": GIVIZEN_TOP},
+           "expert": {"ff": expert_ff, "limit": 7.0}, "shared": {"ff": shared_ff, "limit": 7.0}}
+    common = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+              "q_temp": {"coef": 0.1, "every": 1024}}
+    kinds = [
+        {"type": "attention", "mlp": mlp, "mixer": {**common, "mask": {"size": GIVIZEN_WINDOWS[0]}}},
+        {"type": "attention_2", "mlp": mlp, "mixer": {**common, "mask": {"size": GIVIZEN_WINDOWS[1]}, "softcap": 50.0}},
+    ]
+    return {"architecture": "Givizen", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "logit_softcap": 30.0, "layers": [kinds[i % 2] for i in range(layers)]}
+
+
+def givizen_costs(config, batch: int, context: float, tokens: int, elem: int) -> tuple[float, float]:
+    """(bytes one decode step has to move, flops of a prefill of ``tokens`` tokens) for a Givizen configuration:
+    every weight that a step touches once (of a layer's experts, the ones that ``batch`` tokens choosing ``top`` of
+    them at random are expected to hit), each request's keys and values inside the layer's window; products at two
+    flops per active weight and token, attention over the keys each token sees."""
+    width, vocab = config.hidden_size, config.vocab_size
+    moved = float(vocab * width * elem)
+    flops = 2.0 * vocab * width
+    for layer in config.raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        mixer = width * (m["heads"] * m["dim"] + m["kv_heads"] * (m["dim"] + m["vdim"]) + m["heads"] * m["vdim"])
+        if layer["type"] == "attention_2":
+            mixer += width * m["heads"]
+        experts, top = mlp["router"]["experts"], mlp["router"]["top"]
+        one = 3 * width * mlp["expert"]["ff"]
+        shared = 3 * width * mlp["shared"]["ff"] if mlp.get("shared") else 0
+        hit = experts * (1.0 - (1.0 - top / experts) ** batch)
+        moved += (mixer + width * experts + shared + hit * one) * elem
+        seen = min(context, m["mask"]["size"])
+        moved += batch * seen * m["kv_heads"] * (m["dim"] + m["vdim"]) * elem
+        flops += 2.0 * tokens * (mixer + width * experts + shared + top * one)
+        window = min(tokens, m["mask"]["size"])
+        pairs = window * (window + 1) / 2 + (tokens - window) * window
+        flops += 2.0 * pairs * m["heads"] * (m["dim"] + m["vdim"])
+    return moved, flops
+
+
 def compare_designs(args) -> int:
-    """``--design polosun``: see the module's text."""
+    """``--design polosun`` or ``--design givizen``: see the module's text."""
     import torch
 
-    from cie_amd.config import PolosunConfig, Qwen2Config
+    from cie_amd.config import GivizenConfig, PolosunConfig, Qwen2Config
     from cie_amd.workloads import SHAPES
 
     elem = 2 if args.dtype == "bf16" else 4
@@ -287,7 +342,8 @@ def compare_designs(args) -> int:
     for name in [n for n in args.design_shapes.split(",") if n]:
         shape = SHAPES[name]
         designs = {
-            "polosun": PolosunConfig.from_hf_config(polosun_raw(shape, layers)),
+            args.design: (PolosunConfig.from_hf_config(polosun_raw(shape, layers)) if args.design == "polosun"
+                          else GivizenConfig.from_hf_config(givizen_raw(shape, layers))),
             "qwen2": Qwen2Config.from_hf_config(dict(shape, num_hidden_layers=layers)),
         }
         out[name] = {}
@@ -295,6 +351,8 @@ def compare_designs(args) -> int:
             def costs(batch, context):
                 if design == "polosun":
                     return polosun_costs(config, batch, context, args.prefill_tokens, elem)
+                if design == "givizen":
+                    return givizen_costs(config, batch, context, args.prefill_tokens, elem)
                 return (decode_bytes(config, layers, batch, context, elem), prefill_flops(config, layers, args.prefill_tokens))
 
             record = {}
@@ -319,11 +377,14 @@ def compare_designs(args) -> int:
                     "frac": round(costs(batch, mean_context)[0] / (taken / steps) / 1e9 / HBM_GBPS, 4)}
             out[name][design] = record
     print(json.dumps({
-        "metric": f"Polosun beside the Qwen2.5 decoder of equal width, feed-forward, vocabulary and {layers} layers",
+        "metric": f"{args.design.capitalize()} beside the Qwen2.5 decoder of equal width, feed-forward, vocabulary and {layers} layers",
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
         "data": "synthetic (seeded uniform-random token ids, random weights N(0, 0.02))",
         "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens, "page_size": PAGE,
-                   "polosun_layers": "retention, latent_attention, rglru in turn, each with a dense feed-forward"},
+                   "design_layers": ("retention, latent_attention, rglru in turn, each with a dense feed-forward"
+                                     if args.design == "polosun" else
+                                     f"attention (window {GIVIZEN_WINDOWS[0]}) and attention_2 (window {GIVIZEN_WINDOWS[1]}) in turn, each "
+                                     f"with {GIVIZEN_EXPERTS} experts, {GIVIZEN_TOP} per token, and a shared expert")},
         "shapes": out,
     }))
     return 0
@@ -350,7 +411,7 @@ def main(argv=None) -> int:
                              "(default 16,64,248; '' for none, as with --no-points)")
     parser.add_argument("--other-shapes", default="7b,14b",
                         help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
-    parser.add_argument("--design", default=None, choices=["polosun"],
+    parser.add_argument("--design", default=None, choices=["polosun", "givizen"],
                         help="instead of the default record: this design beside the Qwen2.5 decoder of equal size")
     parser.add_argument("--design-shapes", default="3b,7b", help="the Qwen2.5 shapes whose sizes the comparison takes")
     parser.add_argument("--design-layers", type=int, default=12, help="layers of both models in the comparison")
