@@ -259,12 +259,17 @@ class CacheManager:
     def tokens_missing(self, request_id: str, upto: int) -> int:
         """What ``request_id`` (admitted or not) would still take of :meth:`free_tokens` to hold ``upto``
         tokens: the pages it lacks in the group where it lacks most, times the page size.  A group that
-        keeps a window never holds more than the window and one step's portion."""
+        keeps a window never holds more than the window and one step's portion, and never again the pages
+        that the window has passed."""
         most = 0
+        held_tokens = self._length.get(request_id, 0)
         for group in self.groups:
             pages = group.allocator.pages_for(upto)
             if group.most_per_request is not None:
-                pages = min(pages, group.most_per_request)
+                # the pages below the window's reach from where the request stands are never asked for again
+                # (a request that decodes behind a long prompt holds its window's pages and needs one more at most)
+                passed = max(0, held_tokens + 1 - group.spec.window) // self.page_size
+                pages = min(pages - passed, group.most_per_request)
             table = group.tables.get(request_id, ())
             most = max(most, pages - sum(1 for page in table if page >= 0))
         return max(0, most) * self.page_size

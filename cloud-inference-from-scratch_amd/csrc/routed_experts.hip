@@ -140,6 +140,11 @@ __device__ __forceinline__ bf16x8 scaled_fragment(const uint4 raw, float w) {
 // v_mfma_f32_16x16x32_bf16 with A = rows of x (lane % 16 the row, lane / 16 the eighth of the 32 k), B = rows of
 // the weight (lane % 16 the result column, the same k): lane (r, g) then holds the results of rows g*4 .. g*4+3 at
 // column r.
+// Loads stand without conditions (addresses past an edge are clamped, what they fetch is zeroed when used), the loads
+// of kUnroll steps of 32 k ahead of the products that use them: a wave has that many cache lines of its weight rows
+// under way at once, which is what a step of few rows, bound by the weights' way from memory, needs.
+constexpr int kUnroll = 4;
+
 template <int RT>
 __global__ void __launch_bounds__(256)
 experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_gate_up,
@@ -171,18 +176,25 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
     floatx4 acc_g[RT], acc_u[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc_g[rt] = acc_u[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const int k = k0 + g * 8;
-        const bool k_ok = k < K;
-        const uint4 zero = uint4{0, 0, 0, 0};
-        const uint4 bg = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wg + k) : zero;
-        const uint4 bu = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wu + k) : zero;
+    for (int k0 = 0; k0 < K; k0 += 32 * kUnroll) {
+        uint4 bg[kUnroll], bu[kUnroll], ax[kUnroll][RT];
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            const uint4 raw = k_ok ? *reinterpret_cast<const uint4*>(x_row[rt] + k) : zero;
-            const bf16x8 af = scaled_fragment(raw, weight[rt]);
-            acc_g[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bg), acc_g[rt], 0, 0, 0);
-            acc_u[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bu), acc_u[rt], 0, 0, 0);
+        for (int u = 0; u < kUnroll; ++u) {
+            const int k = min(k0 + u * 32 + g * 8, K - 8);
+            bg[u] = *reinterpret_cast<const uint4*>(wg + k);
+            bu[u] = *reinterpret_cast<const uint4*>(wu + k);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) ax[u][rt] = *reinterpret_cast<const uint4*>(x_row[rt] + k);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool k_ok = k0 + u * 32 + g * 8 < K;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const bf16x8 af = scaled_fragment(ax[u][rt], k_ok ? weight[rt] : 0.f);
+                acc_g[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bg[u]), acc_g[rt], 0, 0, 0);
+                acc_u[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bu[u]), acc_u[rt], 0, 0, 0);
+            }
         }
     }
     if (!col_ok) return;
@@ -215,21 +227,35 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
     const int K = a.ff;
     const bool col_ok = c0 + r < a.hidden;
     const bf16_t* wd = w_down + (static_cast<size_t>(expert) * a.hidden + min(c0 + r, a.hidden - 1)) * K;
+    const bf16_t* a_row[RT];
+    bool row_ok[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        row_ok[rt] = rt * 16 + r < rows;
+        a_row[rt] = act + static_cast<size_t>(begin + min(rt * 16 + r, rows - 1)) * K;
+    }
     floatx4 acc[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const int k = k0 + g * 8;
-        const bool k_ok = k < K;
-        const uint4 zero = uint4{0, 0, 0, 0};
-        const uint4 b = (k_ok && col_ok) ? *reinterpret_cast<const uint4*>(wd + k) : zero;
+    const uint4 zero = uint4{0, 0, 0, 0};
+    for (int k0 = 0; k0 < K; k0 += 32 * kUnroll) {
+        uint4 b[kUnroll], ax[kUnroll][RT];
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            const int row = rt * 16 + r;
-            const uint4 raw = (k_ok && row < rows)
-                ? *reinterpret_cast<const uint4*>(act + static_cast<size_t>(begin + row) * K + k) : zero;
-            acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw),
-                                                              __builtin_bit_cast(bf16x8, b), acc[rt], 0, 0, 0);
+        for (int u = 0; u < kUnroll; ++u) {
+            const int k = min(k0 + u * 32 + g * 8, K - 8);
+            b[u] = *reinterpret_cast<const uint4*>(wd + k);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) ax[u][rt] = *reinterpret_cast<const uint4*>(a_row[rt] + k);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool k_ok = k0 + u * 32 + g * 8 < K;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const uint4 raw = (k_ok && row_ok[rt]) ? ax[u][rt] : zero;
+                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw),
+                                                                  __builtin_bit_cast(bf16x8, b[u]), acc[rt], 0, 0, 0);
+            }
         }
     }
     if (!col_ok) return;

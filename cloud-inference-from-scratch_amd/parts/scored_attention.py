@@ -163,8 +163,7 @@ class ScoredAttention(Part):
                                                  batch.sequences, batch.seq_slot, batch.seq_start, batch.seq_q_len,
                                                  batch.q_start_loc, batch.tokens, h, g, self.kernel_dim,
                                                  self.kernel_vdim, 1, least, **shape)
-            most = 4 if max(self.mfma_dims) <= 64 else 2
-            row_tiles = max(least, most if batch.max_q_len * group > 16 else 1)
+            row_tiles = max(least, 4 if batch.max_q_len * group > 16 else 1)
             while row_tiles > least and -(-batch.tokens * group // (16 * row_tiles)) * g < ops.compute_units():
                 row_tiles //= 2  # (fewer rows a tile where the tiles would not fill the compute units)
             per_tile = (16 * row_tiles) // group

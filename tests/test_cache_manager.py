@@ -243,6 +243,22 @@ def test_window_pool_is_sized_by_window_not_by_context():
     assert m.groups[0].allocator.total_pages == 2 * (6 + 1)
 
 
+def test_a_request_behind_its_window_is_not_counted_as_missing_the_pages_it_gave_back():
+    """Two window groups beside each other: a request that decodes behind a long prompt holds its windows' pages
+    and lacks one more at most, in either group (counted as lacking a window and a portion again, six such requests
+    kept two newcomers waiting for good although the pools had room)."""
+    m = manager(unit_specs=[PagedKV(1, 8, window=64), PagedKV(1, 8, window=256)], kv_tokens=4096, max_running=4,
+                max_model_len=1024, prefill_chunk=128, page_size=16)
+    m.admit("a")
+    assert m.tokens_missing("a", 600) == ((256 + 128) // 16 + 1) * 16         # the larger window, a portion and a page
+    for length in (128, 256, 384, 512, 600):
+        m.ensure_capacity_batch({"a": length})
+        m.commit_lengths({"a": length})
+    assert m.tokens_missing("a", 601) == 0 and m.tokens_missing("a", 609) == 16
+    assert m.tokens_missing("b", 50) == 64                                    # a newcomer: all its pages
+    m.assert_invariants()
+
+
 def test_fixed_state_units_take_no_pages_and_disable_prefix_reuse():
     m = manager(unit_specs=[FixedState((4, 8)), PagedKV(2, 16)], prefix_cache_pages=8)
     assert m.state_units == {0: FixedState((4, 8))} and m.unit_group == {1: 0}
