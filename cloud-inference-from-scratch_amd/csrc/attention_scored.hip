@@ -235,7 +235,10 @@ scored_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k
 //   g = lane / 16) then holds, for row r, the scores of keys g*4 .. g*4+3 of each 16-key tile, which is the A-operand
 //   layout of P in  O[row, d] += P[row, key] * V[key, d]  (B = rows of the transposed values).
 // The softmax runs in base 2 (scores, cap, bias and sink are brought there once).  The four waves' running
-// (max, sum, accumulator) meet in LDS, one wave after the other, and all threads write the tile's rows.
+// (max, sum, accumulator) meet in LDS, one wave after the other, and all threads write the tile's rows.  Few tiles
+// over many keys (single tokens behind long windows) have their keys cut into shares, a workgroup each, whose
+// (max, sum, accumulator) a second kernel joins; sink and gate are then applied there.  The accumulator is rescaled
+// only in blocks where some row's maximum moved, and keys are masked only in blocks that reach an edge of some row.
 struct ScoredArgs {
     const bf16_t* q;          // [tokens, q_heads, D]
     const bf16_t* k_pool;
@@ -256,6 +259,10 @@ struct ScoredArgs {
     int page_shift;
     int tokens_per_tile;
     int n_tiles;
+    int n_splits;        // > 1: the keys of a tile in that many shares of keys_per_split (a multiple of 128), one
+    int keys_per_split;  // workgroup each (blockIdx.z); the shares' sums meet in scored_attention_merge_kernel
+    float* part_o;       // [tiles, kv_heads, splits, rows, DV]
+    float* part_ml;      // [tiles, kv_heads, splits, rows, 2]
     ScoreShape shape;
 };
 
@@ -299,7 +306,24 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
 
     const int hi = start + q0 + n_tok;
     const int lo = (window > 0) ? max(0, start + q0 + 1 - window) : 0;
-    const int range_begin = lo & ~(kKeysPerBlock - 1);
+    int range_begin = lo & ~(kKeysPerBlock - 1);
+    int range_end = hi;
+    const int split = blockIdx.z;
+    if (a.n_splits > 1) {
+        range_begin += split * a.keys_per_split;
+        range_end = min(hi, range_begin + a.keys_per_split);
+    }
+    const int first_pos = start + q0;            // position of the tile's first token (its window reaches back furthest)
+    const int last_lo = (window > 0) ? start + q0 + n_tok - window : 0;  // the first key the tile's last token sees
+
+    if (a.n_splits > 1 && range_begin >= range_end) {  // a share without keys: its statistics say so, its sums are never read
+        float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + split) * ROWS * 2;
+        if (threadIdx.x < ROWS) {
+            pml[threadIdx.x * 2] = -INFINITY;
+            pml[threadIdx.x * 2 + 1] = 0.f;
+        }
+        return;
+    }
 
     uint4 qf[RT][NK];
     int row_pos[RT];      // position of the lane's row r of tile rt; -1 for a row that does not exist
@@ -328,7 +352,9 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
         for (int dt = 0; dt < ND; ++dt) o[rt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int kb = range_begin + wave * kKeysPerBlock; kb < hi; kb += STEP) {
+    for (int kb = range_begin + wave * kKeysPerBlock; kb < range_end; kb += STEP) {
+        // every row sees every key of the block: none lies behind the first token, none before the last one's window
+        const bool inner = kb + kKeysPerBlock - 1 <= first_pos && kb >= last_lo && kb + kKeysPerBlock <= range_end;
         floatx4 s[RT][2];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
@@ -371,7 +397,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = kb + kt * 16 + g * 4 + i;
-                    const bool seen = key <= pos && key >= row_lo;
+                    const bool seen = inner || (key <= pos && key >= row_lo && key < range_end);
                     float x = s[rt][kt][i] * scale;
                     if (cap > 0.f) x = cap * fast_tanh(x * inv_cap);
                     x = x * kLog2e - row_slope[rt] * static_cast<float>(pos - key);
@@ -385,6 +411,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
             const float m_new = fmaxf(m_run[rt], block_max);
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_safe);  // m_run = -inf: 0, and l, O are 0 anyway
+            const bool moved = m_new != m_run[rt];
             m_run[rt] = m_new;
             float p_sum = 0.f;
             uint32_t pw[4];
@@ -399,14 +426,16 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
                 pw[kt * 2 + 1] = pack_bf16(p2, p3);
             }
             l_run[rt] = l_run[rt] * alpha + p_sum;
-            // the accumulator's rows are g*4+i, the statistics' row is r: fetch alpha of those rows
-            float alpha_o[4];
+            if (__any(moved)) {
+                // the accumulator's rows are g*4+i, the statistics' row is r: fetch alpha of those rows
+                float alpha_o[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
+                for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
 #pragma unroll
-            for (int dt = 0; dt < ND; ++dt)
+                for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o[rt][dt][i] *= alpha_o[i];
+                    for (int i = 0; i < 4; ++i) o[rt][dt][i] *= alpha_o[i];
+            }
             const bf16x8 p_frag = __builtin_bit_cast(bf16x8, (uint4{pw[0], pw[1], pw[2], pw[3]}));
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
@@ -437,7 +466,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
             float m_all = m_s[0][row];
 #pragma unroll
             for (int w = 1; w < kScoredWaves; ++w) m_all = fmaxf(m_all, m_s[w][row]);
-            if (a.shape.sinks && row < n_rows)
+            if (a.shape.sinks && row < n_rows && a.n_splits == 1)
                 m_all = fmaxf(m_all, a.shape.sinks[kv_head * group + row % group] * kLog2e);
             const float mine = m_s[wave][row];
             own[rt][i] = (mine == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mine - m_all);
@@ -457,6 +486,29 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
                     }
         }
         __syncthreads();
+    }
+    if (a.n_splits > 1) {
+        // this share's (max, sum, accumulator) of every row, for the merge
+        const size_t unit = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + split;
+        float* po = a.part_o + unit * ROWS * DV;
+        float* pml = a.part_ml + unit * ROWS * 2;
+        for (int row = wave; row < n_rows; row += kScoredWaves) {
+            float m_all = m_s[0][row];
+#pragma unroll
+            for (int w = 1; w < kScoredWaves; ++w) m_all = fmaxf(m_all, m_s[w][row]);
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < kScoredWaves; ++w) {
+                const float mine = m_s[w][row];
+                sum += (mine == -INFINITY) ? 0.f : l_s[w][row] * __builtin_amdgcn_exp2f(mine - m_all);
+            }
+            if (lane == 0) {
+                pml[row * 2] = m_all;
+                pml[row * 2 + 1] = sum;
+            }
+            for (int d = lane; d < DV; d += kWave) po[static_cast<size_t>(row) * DV + d] = o_s[row][d];
+        }
+        return;
     }
     for (int row = wave; row < n_rows; row += kScoredWaves) {
         const int tok = row / group;
@@ -485,9 +537,56 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
     }
 }
 
+// Joins the shares of a tile's keys: one workgroup per (tile, kv head), one wave per row in turn.
+__global__ void __launch_bounds__(256) scored_attention_merge_kernel(ScoredArgs a, int rows_per_tile, int DV) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int tile = blockIdx.x;
+    const int kv_head = blockIdx.y;
+    const int group = a.q_heads / a.kv_heads;
+    const int seq = a.tile_seq ? a.tile_seq[tile] : tile;
+    const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
+    const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
+    const int n_rows = n_tok * group;
+    const int first_row_token = a.q_start_loc[seq] + q0;
+    const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
+    for (int row = wave; row < n_rows; row += 4) {
+        const int tok = row / group;
+        const int head = kv_head * group + (row - tok * group);
+        float m_all = -INFINITY;
+        for (int sp = 0; sp < a.n_splits; ++sp) m_all = fmaxf(m_all, a.part_ml[((unit0 + sp) * rows_per_tile + row) * 2]);
+        float den = 0.f;
+        if (a.shape.sinks) {
+            const float sink = a.shape.sinks[head] * kLog2e;
+            m_all = fmaxf(m_all, sink);
+            den = __builtin_amdgcn_exp2f(sink - m_all);
+        }
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};  // DV <= 256: four numbers a lane
+        for (int sp = 0; sp < a.n_splits; ++sp) {
+            const float* ml = a.part_ml + ((unit0 + sp) * rows_per_tile + row) * 2;
+            if (ml[0] == -INFINITY) continue;  // (a share without keys; the same for every lane)
+            const float f = __builtin_amdgcn_exp2f(ml[0] - m_all);
+            den += ml[1] * f;
+            const float* po = a.part_o + ((unit0 + sp) * rows_per_tile + row) * DV;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (lane + i * kWave < DV) acc[i] += po[lane + i * kWave] * f;
+        }
+        float factor = 1.0f / den;
+        if (a.gate) {
+            const float z = to_float(a.gate[static_cast<size_t>(first_row_token + tok) * a.gate_stride + head]);
+            factor *= 1.0f / (1.0f + __expf(-z));
+        }
+        bf16_t* dst = a.out + (static_cast<size_t>(first_row_token + tok) * a.q_heads + head) * DV;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (lane + i * kWave < DV) dst[lane + i * kWave] = from_float<bf16_t>(acc[i] * factor);
+    }
+}
+
 template <int D, int DV>
 int launch_scored(hipStream_t s, const ScoredArgs& a, int row_tiles) {
-    dim3 grid(a.n_tiles, a.kv_heads);
+    dim3 grid(a.n_tiles, a.kv_heads, a.n_splits);
     if (row_tiles == 1)
         scored_attention_mfma_kernel<D, DV, 1><<<grid, 64 * kScoredWaves, 0, s>>>(a);
     else if (row_tiles == 2)
@@ -496,6 +595,9 @@ int launch_scored(hipStream_t s, const ScoredArgs& a, int row_tiles) {
         scored_attention_mfma_kernel<D, DV, 4><<<grid, 64 * kScoredWaves, 0, s>>>(a);
     else
         return CIE_BAD_ARGUMENT;
+    if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
+    if (a.n_splits > 1)
+        scored_attention_merge_kernel<<<dim3(a.n_tiles, a.kv_heads), 256, 0, s>>>(a, 16 * row_tiles, DV);
     return cie_after_launch();
 }
 
@@ -574,14 +676,22 @@ CIE_API int cie_scored_attention_mfma(void* stream, const void* q, const void* k
                                       const int* seq_q_len, const int* q_start_loc, const void* gate,
                                       int gate_stride, void* out, int q_heads, int kv_heads, int D, int DV,
                                       int page_size, int tokens_per_tile, int row_tiles, int window, float scale,
-                                      float softcap, const float* slopes, const float* sinks) {
+                                      float softcap, const float* slopes, const float* sinks, int n_splits,
+                                      int keys_per_split, float* part_o, float* part_ml) {
     if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
         (page_size & (page_size - 1)) || table_width <= 0 || tokens_per_tile < 1 || kv_heads > 65535 ||
         (tile_seq == nullptr) != (tile_q0 == nullptr) || (gate && gate_stride < q_heads))
         return CIE_BAD_ARGUMENT;
     if (tokens_per_tile * (q_heads / kv_heads) > 16 * row_tiles) return CIE_BAD_ARGUMENT;
+    if (n_splits < 1 || n_splits > 65535 ||
+        (n_splits > 1 && (keys_per_split < 128 || keys_per_split % 128 || !part_o || !part_ml || DV > 256)))
+        return CIE_BAD_ARGUMENT;
     if (n_tiles == 0) return CIE_OK;
     ScoredArgs a;
+    a.n_splits = n_splits;
+    a.keys_per_split = keys_per_split;
+    a.part_o = part_o;
+    a.part_ml = part_ml;
     a.q = static_cast<const bf16_t*>(q);
     a.k_pool = static_cast<const bf16_t*>(k_pool);
     a.v_pool = static_cast<const bf16_t*>(v_pool);

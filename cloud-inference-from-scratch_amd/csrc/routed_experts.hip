@@ -11,9 +11,12 @@
 //   down       parts[p, :] = W_down[e] act[i, :], float32, one row per pair: whoever adds the branch sums a
 //              token's `top` rows, in a fixed order.
 //
-// bfloat16 with widths that are multiples of 8 runs on the matrix cores (four waves a workgroup, each a tile of 16
-// columns over all of K for up to 16 * RT rows); anything else takes the plain form of one thread per result, whose
-// sums run over k in order, float32.  Weights: gate_up [experts, 2 * ff, hidden] (gate rows first), down
+// bfloat16 with widths that are multiples of 8 runs on the matrix cores, in one of two forms.  Few rows an expert (a
+// decode step): four waves a workgroup, each a tile of 16 columns over all of K for up to 16 * RT rows, operands
+// straight from memory.  Many rows an expert (a prompt's portion): the rows are first gathered in sorted order and
+// multiplied by their weights (`gather`), then tiles of 128 rows x 128 columns a workgroup, slices of 64 k staged
+// through LDS in the operand order of the matrix instruction, the next slice's loads under way while this one is
+// multiplied.  Anything else takes the plain form of one thread per result, whose sums run over k in order, float32.  Weights: gate_up [experts, 2 * ff, hidden] (gate rows first), down
 // [experts, hidden, ff].
 #include "activation_forms.h"
 #include "attention_args.h"
@@ -268,6 +271,155 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
         }
 }
 
+
+// ---- many rows an expert: tiles of 128 x 128 through LDS ---------------------------------------------------------
+// A slice of 64 k of 128 operand rows lies in LDS as two halves of 32 k, each [128 rows][32 k] (64 bytes a row): the
+// 16 rows x 64 bytes that the 64 lanes of one matrix instruction read are 1 KB in a row, so the reads meet no bank
+// twice; a thread stages 16 bytes of rows t / 8 + 32 j, and a wave's stores are 512 bytes in a row per half.
+// Wave w of four owns rows 64 (w / 2) .. and the column half w % 2: 4 x 4 products of 16 x 16 per 32 k.
+constexpr int kTile = 128;
+constexpr int kSlice = 64;
+
+// xs[i, :] = bf16(weight(pair) * x[token(pair), :]) for the i-th pair of the sorted order.
+__global__ void __launch_bounds__(256)
+experts_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xs, const int* __restrict__ sorted,
+                      const float* __restrict__ pair_weight, int pairs, int top, int hidden) {
+    const int place = blockIdx.x;
+    const int pair = sorted[place];
+    const float w = pair_weight[pair];
+    const bf16_t* src = x + static_cast<size_t>(pair / top) * hidden;
+    bf16_t* dst = xs + static_cast<size_t>(place) * hidden;
+    for (int k = threadIdx.x * 8; k < hidden; k += blockDim.x * 8) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + k);
+        *reinterpret_cast<uint4*>(dst + k) = __builtin_bit_cast(uint4, scaled_fragment(raw, w));
+    }
+}
+
+// GATE_UP: a[rows, K] x (gate rows | up rows of 64 result columns) -> act = unit(gate, up), bfloat16.
+// else:    a[rows, K] x 128 rows of the down weight -> parts[pair], float32.
+template <bool GATE_UP>
+__global__ void __launch_bounds__(256)
+experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict__ weight, bf16_t* __restrict__ act,
+                     float* __restrict__ parts, ExpertArgs a) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][2][kTile * 32];
+    __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][2][kTile * 32];
+    const int tile = blockIdx.x;
+    if (tile >= *a.n_tiles) return;
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int expert = a.tile_expert[tile];
+    const int begin = a.tile_begin[tile];
+    const int rows = a.tile_count[tile];
+    const int K = GATE_UP ? a.hidden : a.ff;
+    const int n_out = GATE_UP ? a.ff : a.hidden;            // result columns of the expert
+    const int cols_here = GATE_UP ? kTile / 2 : kTile;      // ... of which this workgroup makes so many
+    const int c0 = blockIdx.y * cols_here;
+    // staging: thread t brings 16 bytes (8 k) of rows t / 8 + 32 j, j = 0..3, for A and for B
+    const int s_row = threadIdx.x / 8;
+    const int s_k = (threadIdx.x % 8) * 8;
+    const bf16_t* a_src[4];
+    const bf16_t* b_src[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = s_row + 32 * j;
+        a_src[j] = a_rows + static_cast<size_t>(begin + min(row, rows - 1)) * K;
+        // weight row of staged row `row`: GATE_UP lays the workgroup's columns out as [half][gate 32 | up 32]
+        int col;
+        if (GATE_UP) {
+            const int half = row / 64, within = row % 64;
+            col = c0 + half * 32 + (within % 32);
+            col = min(col, n_out - 1) + (within >= 32 ? n_out : 0);
+        } else {
+            col = min(c0 + row, n_out - 1);
+        }
+        b_src[j] = weight + (static_cast<size_t>(expert) * (GATE_UP ? 2 * n_out : n_out) + col) * K;
+    }
+    const int s_at = (s_k / 32) * (kTile * 32) + (s_k % 32);   // + row * 32: place in a staged slice
+    uint4 ra[4], rb[4];
+    auto fetch = [&](int k0) {
+        const int k = min(k0 + s_k, K - 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ra[j] = *reinterpret_cast<const uint4*>(a_src[j] + k);
+            rb[j] = *reinterpret_cast<const uint4*>(b_src[j] + k);
+        }
+    };
+    auto stage = [&](int buffer, int k0) {
+        const bool k_ok = k0 + s_k < K;                         // (a slice past the end of K holds zeros on the A side)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int at = s_at + (s_row + 32 * j) * 32;
+            *reinterpret_cast<uint4*>(&lds_a[buffer][0][0] + at) = k_ok ? ra[j] : uint4{0, 0, 0, 0};
+            *reinterpret_cast<uint4*>(&lds_b[buffer][0][0] + at) = rb[j];
+        }
+    };
+    floatx4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int row0 = (wave / 2) * 64;
+    const int col0 = (wave % 2) * 64;
+    fetch(0);
+    stage(0, 0);
+    __syncthreads();
+    int buffer = 0;
+    for (int k0 = 0; k0 < K; k0 += kSlice) {
+        const bool more = k0 + kSlice < K;
+        if (more) fetch(k0 + kSlice);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            bf16x8 af[4], bfr[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buffer][half][(row0 + i * 16 + r) * 32 + g * 8]);
+                bfr[i] = *reinterpret_cast<const bf16x8*>(&lds_b[buffer][half][(col0 + i * 16 + r) * 32 + g * 8]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stage(buffer ^ 1, k0 + kSlice);
+        __syncthreads();
+        buffer ^= 1;
+    }
+    // lane (r, g) holds rows g*4 .. g*4+3 of row tile i at column r of column tile j
+    if (GATE_UP) {
+        // the wave's 64 staged columns are [gate 32 | up 32] of result columns c0 + (wave % 2) * 32 ..
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = c0 + (wave % 2) * 32 + j * 16 + r;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int row = row0 + i * 16 + g * 4 + v;
+                    if (row < rows && col < n_out)
+                        act[static_cast<size_t>(begin + row) * n_out + col] =
+                            from_float<bf16_t>(clamped_glu(acc[i][j][v], acc[i][j + 2][v], a.limit, a.alpha, a.offset));
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = row0 + i * 16 + g * 4 + v;
+                if (row >= rows) continue;
+                float* dst = parts + static_cast<size_t>(a.sorted[begin + row]) * n_out;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int col = c0 + col0 + j * 16 + r;
+                    if (col < n_out) dst[col] = acc[i][j][v];
+                }
+            }
+    }
+}
+
 // The plain forms: tiles of up to 16 rows, 16 columns a workgroup, one thread per result.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -345,6 +497,10 @@ CIE_API int cie_experts_gate_up(void* stream, int dtype, int mfma, const void* x
         const bf16_t* xs = static_cast<const bf16_t*>(x);
         const bf16_t* ws = static_cast<const bf16_t*>(w_gate_up);
         bf16_t* as = static_cast<bf16_t*>(act);
+        if (tile_rows == kTile) {  // (x: the rows gathered in sorted order, weights applied)
+            experts_tiled_kernel<true><<<dim3(max_tiles, (ff + 63) / 64), 256, 0, s>>>(xs, ws, as, nullptr, a);
+            return cie_after_launch();
+        }
         if (tile_rows == 16) experts_gate_up_mfma_kernel<1><<<grid, 256, 0, s>>>(xs, ws, as, a);
         else if (tile_rows == 32) experts_gate_up_mfma_kernel<2><<<grid, 256, 0, s>>>(xs, ws, as, a);
         else if (tile_rows == 64) experts_gate_up_mfma_kernel<4><<<grid, 256, 0, s>>>(xs, ws, as, a);
@@ -377,6 +533,10 @@ CIE_API int cie_experts_down(void* stream, int dtype, int mfma, const void* act,
         dim3 grid(max_tiles, (hidden + 63) / 64);
         const bf16_t* as = static_cast<const bf16_t*>(act);
         const bf16_t* ws = static_cast<const bf16_t*>(w_down);
+        if (tile_rows == kTile) {
+            experts_tiled_kernel<false><<<dim3(max_tiles, (hidden + kTile - 1) / kTile), 256, 0, s>>>(as, ws, nullptr, parts, a);
+            return cie_after_launch();
+        }
         if (tile_rows == 16) experts_down_mfma_kernel<1><<<grid, 256, 0, s>>>(as, ws, parts, a);
         else if (tile_rows == 32) experts_down_mfma_kernel<2><<<grid, 256, 0, s>>>(as, ws, parts, a);
         else if (tile_rows == 64) experts_down_mfma_kernel<4><<<grid, 256, 0, s>>>(as, ws, parts, a);
@@ -391,5 +551,16 @@ CIE_API int cie_experts_down(void* stream, int dtype, int mfma, const void* act,
         experts_down_plain_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(act), static_cast<const bf16_t*>(w_down), parts, a);
     else
         return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// xs [pairs, hidden]: row i is the input row of the i-th sorted pair times the pair's weight (bfloat16, hidden a
+// multiple of 8): what the tiled form of cie_experts_gate_up takes as x.
+CIE_API int cie_experts_gather(void* stream, const void* x, void* xs, const int* sorted, const float* pair_weight,
+                               int pairs, int top, int hidden) {
+    if (pairs < 0 || top < 1 || hidden < 8 || hidden % 8) return CIE_BAD_ARGUMENT;
+    if (pairs == 0) return CIE_OK;
+    experts_gather_kernel<<<pairs, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xs), sorted, pair_weight, pairs, top, hidden);
     return cie_after_launch();
 }

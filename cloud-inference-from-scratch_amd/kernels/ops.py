@@ -1245,10 +1245,13 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
                           q_start_loc: torch.Tensor, tokens: int, q_heads: int, kv_heads: int, dim: int, vdim: int,
                           tokens_per_tile: int, row_tiles: int, window: Optional[int], scale: float,
                           softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
-                          sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                          n_splits: int = 1, keys_per_split: int = 0) -> torch.Tensor:
     """The same on the matrix cores (bfloat16, (dim, vdim) in ``SCORED_MFMA_DIMS``, pages of a power of two >= 4):
     tiles of ``tokens_per_tile`` consecutive tokens of one sequence (``tile_seq``, ``tile_q0`` int32 [n_tiles]; both
-    ``None``: tile i is sequence i's first), whose rows times the heads per key head fill ``row_tiles`` tiles of 16."""
+    ``None``: tile i is sequence i's first), whose rows times the heads per key head fill ``row_tiles`` tiles of 16.
+    ``n_splits > 1``: every tile's keys in that many shares of ``keys_per_split`` (a multiple of 128; the shares must
+    cover the longest range of keys a tile sees), a workgroup each, joined by a second kernel."""
     _gpu("q", q, torch.bfloat16, 2)
     if not (q.shape == (tokens, q_heads * dim) and q_heads % kv_heads == 0 and (dim, vdim) in SCORED_MFMA_DIMS):
         raise ValueError(f"q {tuple(q.shape)} / heads of {dim}, {vdim} are not what the matrix-core form takes")
@@ -1277,17 +1280,27 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
     _check_score_shape(q_heads, slopes, sinks, softcap)
     gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
     out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
+    part_o = part_ml = None
+    if n_splits > 1:
+        if keys_per_split < 128 or keys_per_split % 128:
+            raise ValueError(f"shares of the keys are multiples of 128, got {keys_per_split}")
+        units = n_tiles * kv_heads * n_splits * 16 * row_tiles
+        part_o = torch.empty(units * vdim, dtype=torch.float32, device=q.device)
+        part_ml = torch.empty(units * 2, dtype=torch.float32, device=q.device)
+    elif n_splits != 1:
+        raise ValueError("n_splits must be positive")
     _run("cie_scored_attention_mfma", load_library().cie_scored_attention_mfma(
         _stream(), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _i(block_table.shape[1]), _ptr(tile_seq),
         _ptr(tile_q0), _i(n_tiles), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len), _ptr(q_start_loc), _ptr(gate),
         _i(gate_stride), _ptr(out), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(tokens_per_tile),
-        _i(row_tiles), _i(window or 0), _f(scale), _f(softcap or 0.0), _ptr(slopes), _ptr(sinks)))
+        _i(row_tiles), _i(window or 0), _f(scale), _f(softcap or 0.0), _ptr(slopes), _ptr(sinks), _i(n_splits),
+        _i(keys_per_split), _ptr(part_o), _ptr(part_ml)))
     return out
 
 
 # ---------------------------------------------------------------------------
 MAX_EXPERTS = 1024
-EXPERT_TILE_ROWS = (16, 32, 64)  # rows of one expert that a workgroup of the matrix-core forms takes
+EXPERT_TILE_ROWS = (16, 32, 64, 128)  # rows of one expert that a workgroup of the matrix-core forms takes (128: through LDS)
 
 
 class ExpertRoute:
@@ -1337,12 +1350,18 @@ def experts_forward(x: torch.Tensor, route: ExpertRoute, w_gate_up: torch.Tensor
             and tokens * route.top == route.pairs):
         raise ValueError(f"expert weights {tuple(w_gate_up.shape)}, {tuple(w_down.shape)} do not fit rows {tuple(x.shape)}")
     if mfma and not (x.dtype == torch.bfloat16 and hidden % 8 == 0 and ff % 8 == 0 and route.tile_rows in EXPERT_TILE_ROWS):
-        raise ValueError("the matrix-core form takes bfloat16, widths that are multiples of 8 and tiles of 16, 32 or 64 rows")
+        raise ValueError("the matrix-core form takes bfloat16, widths that are multiples of 8 and tiles of 16, 32, 64 or 128 rows")
     if not mfma and route.tile_rows > 16:
         raise ValueError("the plain form takes tiles of up to 16 rows")
     act = torch.empty((route.pairs, ff), dtype=x.dtype, device=x.device)
     parts = torch.empty((tokens, route.top, hidden), dtype=torch.float32, device=x.device)
     lib = load_library()
+    if mfma and route.tile_rows == 128:
+        # many rows an expert: the rows in sorted order, weights applied, for the form that stages tiles through LDS
+        gathered = torch.empty((route.pairs, hidden), dtype=x.dtype, device=x.device)
+        _run("cie_experts_gather", lib.cie_experts_gather(_stream(), _ptr(x), _ptr(gathered), _ptr(route.sorted),
+                                                          _ptr(route.pair_weight), _i(route.pairs), _i(route.top), _i(hidden)))
+        x = gathered
     _run("cie_experts_gate_up", lib.cie_experts_gate_up(
         _stream(), _i(_code(x.dtype)), _i(1 if mfma else 0), _ptr(x), _ptr(w_gate_up), _ptr(act), _ptr(route.sorted),
         _ptr(route.pair_weight), _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count),

@@ -83,7 +83,7 @@ class RoutedExperts(Part):
         if not self.mfma:
             return 16
         mean = tokens * self.top / self.experts
-        return 64 if mean > 32 else 32 if mean > 16 else 16
+        return 128 if mean > 48 else 64 if mean > 32 else 32 if mean > 16 else 16
 
     def forward(self, x: torch.Tensor):
         tokens = x.shape[0]

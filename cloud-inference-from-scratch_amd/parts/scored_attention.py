@@ -157,12 +157,25 @@ class ScoredAttention(Part):
         if q.dtype == torch.bfloat16 and self.mfma_dims and group <= 64 and page_size >= 4 and not page_size & (page_size - 1):
             # rows of a tile: a token's heads of one key head, and as many tokens as fill the tile
             least = 1 if group <= 16 else 2 if group <= 32 else 4
+            # the most keys a token sees in this step (a captured step: in any of its replays)
+            bound = batch.static_plan.max_keys if batch.static_plan is not None else batch.max_context
+            bound = bound if self.window is None else min(bound, self.window)
+
+            def shares(tiles: int, span: int) -> dict:
+                """Few tiles over many keys: the keys in shares of at least 128, about two workgroups a compute unit."""
+                reach = bound + span + 32                        # a tile's range starts at a multiple of 32
+                wanted = min(2 * ops.compute_units() // max(tiles * g, 1), reach // 128)
+                if wanted < 2:
+                    return {}
+                per = -(-(-(-reach // wanted)) // 128) * 128
+                return dict(n_splits=-(-reach // per), keys_per_split=per)
+
             if batch.static_plan is not None and batch.static_plan.decode_rows in (None, batch.sequences):
                 # a captured step of single tokens: tile i is sequence i, nothing comes from the host
                 return ops.scored_attention_mfma(q, view.k_pool, view.v_pool, view.block_table, None, None,
                                                  batch.sequences, batch.seq_slot, batch.seq_start, batch.seq_q_len,
                                                  batch.q_start_loc, batch.tokens, h, g, self.kernel_dim,
-                                                 self.kernel_vdim, 1, least, **shape)
+                                                 self.kernel_vdim, 1, least, **shape, **shares(batch.sequences, 1))
             row_tiles = max(least, 4 if batch.max_q_len * group > 16 else 1)
             while row_tiles > least and -(-batch.tokens * group // (16 * row_tiles)) * g < ops.compute_units():
                 row_tiles //= 2  # (fewer rows a tile where the tiles would not fill the compute units)
@@ -171,7 +184,7 @@ class ScoredAttention(Part):
             return ops.scored_attention_mfma(q, view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0, n_tiles,
                                              batch.seq_slot, batch.seq_start, batch.seq_q_len, batch.q_start_loc,
                                              batch.tokens, h, g, self.kernel_dim, self.kernel_vdim, per_tile,
-                                             row_tiles, **shape)
+                                             row_tiles, **shape, **shares(n_tiles, per_tile))
         if q.dtype == torch.bfloat16 and (self.kernel_dim, self.kernel_vdim, group, page_size) not in _SAID_GENERIC:
             _SAID_GENERIC.add((self.kernel_dim, self.kernel_vdim, group, page_size))
             warnings.warn(f"bfloat16 attention with heads of {self.head_dim} and {self.value_dim} numbers, {group} query "

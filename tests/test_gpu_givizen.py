@@ -387,6 +387,12 @@ def test_attention_kernels_against_the_plain_scores(shape, dtype):
                                                 dev([1]), dev([first]), dev([count]), dev([0, count]), count, H, G, D, V,
                                                 per_tile, row_tiles, **common)
                 assert torch.allclose(got.double().cpu().reshape(count, H, V), want[rows], atol=tol, rtol=tol), (use, first, "mfma")
+                # the same with every tile's keys in shares of 128, joined by the second kernel
+                reach = min(first + count, window) + per_tile + 32
+                got = ops.scored_attention_mfma(qd, k_pool, v_pool, table, dev([0] * len(firsts)), dev(firsts), len(firsts),
+                                                dev([1]), dev([first]), dev([count]), dev([0, count]), count, H, G, D, V,
+                                                per_tile, row_tiles, **common, n_splits=-(-reach // 128), keys_per_split=128)
+                assert torch.allclose(got.double().cpu().reshape(count, H, V), want[rows], atol=tol, rtol=tol), (use, first, "shares")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -444,7 +450,7 @@ def test_routed_experts_kernels(sizes, dtype):
     gate_up = torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(E)]).to(dtype).cuda()
     down = torch.stack([w[f"e{e}.down"] for e in range(E)]).to(dtype).cuda()
     mfma = dtype == torch.bfloat16 and width % 8 == 0 and ff % 8 == 0
-    for tile_rows in ((16, 32, 64) if mfma else (16, 5)):
+    for tile_rows in ((16, 32, 64, 128) if mfma else (16, 5)):
         route = ops.experts_route(logits.cuda(), top, tile_rows)
         scores = torch.sigmoid(logits)
         want_w, want_e = torch.topk(scores, top, dim=1)
