@@ -537,7 +537,11 @@ __global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kerne
     }
 }
 
-// Joins the shares of a tile's keys: one workgroup per (tile, kv head), one wave per row in turn.
+// Joins the shares of a tile's keys: one wave per row (four rows a workgroup).  Lane s fetches the statistics of share
+// s (and s + 64, ...), so the common reference and every share's factor are known after one round of loads; the shares'
+// sums are then fetched without waiting on one another.
+constexpr int kMergeShares = 64;  // shares whose factors one pass keeps in a lane each
+
 __global__ void __launch_bounds__(256) scored_attention_merge_kernel(ScoredArgs a, int rows_per_tile, int DV) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -548,40 +552,49 @@ __global__ void __launch_bounds__(256) scored_attention_merge_kernel(ScoredArgs 
     const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     const int n_rows = n_tok * group;
+    const int row = blockIdx.z * 4 + wave;
+    if (row >= n_rows) return;
     const int first_row_token = a.q_start_loc[seq] + q0;
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
-    for (int row = wave; row < n_rows; row += 4) {
-        const int tok = row / group;
-        const int head = kv_head * group + (row - tok * group);
-        float m_all = -INFINITY;
-        for (int sp = 0; sp < a.n_splits; ++sp) m_all = fmaxf(m_all, a.part_ml[((unit0 + sp) * rows_per_tile + row) * 2]);
-        float den = 0.f;
-        if (a.shape.sinks) {
-            const float sink = a.shape.sinks[head] * kLog2e;
-            m_all = fmaxf(m_all, sink);
-            den = __builtin_amdgcn_exp2f(sink - m_all);
+    const int tok = row / group;
+    const int head = kv_head * group + (row - tok * group);
+    float m_all = -INFINITY;
+    for (int sp = lane; sp < a.n_splits; sp += kWave)
+        m_all = fmaxf(m_all, a.part_ml[((unit0 + sp) * rows_per_tile + row) * 2]);
+    m_all = wave_max(m_all);
+    float sink_term = 0.f;  // the sink's share of the denominator, counted once
+    if (a.shape.sinks) {
+        const float sink = a.shape.sinks[head] * kLog2e;
+        m_all = fmaxf(m_all, sink);
+        sink_term = __builtin_amdgcn_exp2f(sink - m_all);
+    }
+    float den = 0.f;        // this lane's shares of it
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};  // DV <= 256: four numbers a lane
+    for (int base = 0; base < a.n_splits; base += kMergeShares) {
+        float mine = 0.f;  // the factor of share base + lane; 0 for a share without keys
+        if (base + lane < a.n_splits) {
+            const float* ml = a.part_ml + ((unit0 + base + lane) * rows_per_tile + row) * 2;
+            mine = (ml[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m_all);
+            den += ml[1] * mine;
         }
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};  // DV <= 256: four numbers a lane
-        for (int sp = 0; sp < a.n_splits; ++sp) {
-            const float* ml = a.part_ml + ((unit0 + sp) * rows_per_tile + row) * 2;
-            if (ml[0] == -INFINITY) continue;  // (a share without keys; the same for every lane)
-            const float f = __builtin_amdgcn_exp2f(ml[0] - m_all);
-            den += ml[1] * f;
-            const float* po = a.part_o + ((unit0 + sp) * rows_per_tile + row) * DV;
+        const int count = min(kMergeShares, a.n_splits - base);
+        for (int sp = 0; sp < count; ++sp) {
+            const float f = __shfl(mine, sp, kWave);
+            const float* po = a.part_o + ((unit0 + base + sp) * rows_per_tile + row) * DV;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (lane + i * kWave < DV) acc[i] += po[lane + i * kWave] * f;
+                if (lane + i * kWave < DV) acc[i] = fmaf(f == 0.f ? 0.f : po[lane + i * kWave], f, acc[i]);
         }
-        float factor = 1.0f / den;
-        if (a.gate) {
-            const float z = to_float(a.gate[static_cast<size_t>(first_row_token + tok) * a.gate_stride + head]);
-            factor *= 1.0f / (1.0f + __expf(-z));
-        }
-        bf16_t* dst = a.out + (static_cast<size_t>(first_row_token + tok) * a.q_heads + head) * DV;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (lane + i * kWave < DV) dst[lane + i * kWave] = from_float<bf16_t>(acc[i] * factor);
     }
+    float factor = 1.0f / (wave_sum(den) + sink_term);
+    if (a.gate) {
+        const float z = to_float(a.gate[static_cast<size_t>(first_row_token + tok) * a.gate_stride + head]);
+        factor *= 1.0f / (1.0f + __expf(-z));
+    }
+    bf16_t* dst = a.out + (static_cast<size_t>(first_row_token + tok) * a.q_heads + head) * DV;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (lane + i * kWave < DV) dst[lane + i * kWave] = from_float<bf16_t>(acc[i] * factor);
 }
 
 template <int D, int DV>
@@ -597,7 +610,7 @@ int launch_scored(hipStream_t s, const ScoredArgs& a, int row_tiles) {
         return CIE_BAD_ARGUMENT;
     if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
     if (a.n_splits > 1)
-        scored_attention_merge_kernel<<<dim3(a.n_tiles, a.kv_heads), 256, 0, s>>>(a, 16 * row_tiles, DV);
+        scored_attention_merge_kernel<<<dim3(a.n_tiles, a.kv_heads, 4 * row_tiles), 256, 0, s>>>(a, 16 * row_tiles, DV);
     return cie_after_launch();
 }
 

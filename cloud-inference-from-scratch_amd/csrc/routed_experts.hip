@@ -273,9 +273,10 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
 
 
 // ---- many rows an expert: tiles of 128 x 128 through LDS ---------------------------------------------------------
-// A slice of 64 k of 128 operand rows lies in LDS as two halves of 32 k, each [128 rows][32 k] (64 bytes a row): the
-// 16 rows x 64 bytes that the 64 lanes of one matrix instruction read are 1 KB in a row, so the reads meet no bank
-// twice; a thread stages 16 bytes of rows t / 8 + 32 j, and a wave's stores are 512 bytes in a row per half.
+// A slice of 64 k of 128 operand rows lies in LDS as [128 rows][8 pieces of 8 k], piece p of row m at place
+// p ^ ((m >> 1) & 7) of the row: the sixteen lanes that the hardware serves together then touch every bank once, both
+// when a matrix instruction's operand is read (rows m .. m + 15, one piece) and when a slice is staged (two rows,
+// all their pieces; a thread stages 16 bytes of rows t / 8 + 32 j, which it fetched as whole cache lines a row).
 // Wave w of four owns rows 64 (w / 2) .. and the column half w % 2: 4 x 4 products of 16 x 16 per 32 k.
 constexpr int kTile = 128;
 constexpr int kSlice = 64;
@@ -301,8 +302,8 @@ template <bool GATE_UP>
 __global__ void __launch_bounds__(256)
 experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict__ weight, bf16_t* __restrict__ act,
                      float* __restrict__ parts, ExpertArgs a) {
-    __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][2][kTile * 32];
-    __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][2][kTile * 32];
+    __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][kTile * kSlice];
+    __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][kTile * kSlice];
     const int tile = blockIdx.x;
     if (tile >= *a.n_tiles) return;
     const int lane = threadIdx.x % kWave;
@@ -336,7 +337,7 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
         }
         b_src[j] = weight + (static_cast<size_t>(expert) * (GATE_UP ? 2 * n_out : n_out) + col) * K;
     }
-    const int s_at = (s_k / 32) * (kTile * 32) + (s_k % 32);   // + row * 32: place in a staged slice
+    auto place = [](int row, int piece) { return row * kSlice + ((piece ^ ((row >> 1) & 7)) << 3); };
     uint4 ra[4], rb[4];
     auto fetch = [&](int k0) {
         const int k = min(k0 + s_k, K - 8);
@@ -350,9 +351,9 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
         const bool k_ok = k0 + s_k < K;                         // (a slice past the end of K holds zeros on the A side)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int at = s_at + (s_row + 32 * j) * 32;
-            *reinterpret_cast<uint4*>(&lds_a[buffer][0][0] + at) = k_ok ? ra[j] : uint4{0, 0, 0, 0};
-            *reinterpret_cast<uint4*>(&lds_b[buffer][0][0] + at) = rb[j];
+            const int at = place(s_row + 32 * j, s_k >> 3);
+            *reinterpret_cast<uint4*>(&lds_a[buffer][at]) = k_ok ? ra[j] : uint4{0, 0, 0, 0};
+            *reinterpret_cast<uint4*>(&lds_b[buffer][at]) = rb[j];
         }
     };
     floatx4 acc[4][4];
@@ -374,8 +375,8 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
             bf16x8 af[4], bfr[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buffer][half][(row0 + i * 16 + r) * 32 + g * 8]);
-                bfr[i] = *reinterpret_cast<const bf16x8*>(&lds_b[buffer][half][(col0 + i * 16 + r) * 32 + g * 8]);
+                af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buffer][place(row0 + i * 16 + r, half * 4 + g)]);
+                bfr[i] = *reinterpret_cast<const bf16x8*>(&lds_b[buffer][place(col0 + i * 16 + r, half * 4 + g)]);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
