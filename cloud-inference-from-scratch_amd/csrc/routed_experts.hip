@@ -1,8 +1,9 @@
 // A feed-forward of many small gated experts of which every token uses a few.
 //
-//   route      s = sigmoid(z) for float32 router logits z [tokens, experts]; the `top` largest are chosen (the
-//              lowest index wins a tie); a (token, choice) *pair* p = token * top + k gets the expert and the
-//              score as it is (not renormalised).
+//   route      s = sigmoid(z) for float32 router logits z [tokens, experts]; the `top` largest are chosen, ranked
+//              by z itself (s rises with z, but two large z can round to one s; the lowest index wins a tie);
+//              a (token, choice) *pair* p = token * top + k gets the expert and the score as it is (not
+//              renormalised).
 //   arrange    pairs sorted by expert and cut into tiles of at most `tile_rows` rows of one expert; everything the
 //              later kernels need stays on the device (the count of tiles too), so a step can be captured: grids
 //              are sized for the most tiles there can be, and workgroups past the count leave at once.
@@ -39,17 +40,20 @@ route_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
     const float* z = logits + static_cast<size_t>(token) * experts;
     constexpr int kMine = kMaxExperts / kWave;
     float mine[kMine];
+    unsigned out = 0;  // bit i: expert lane + i * kWave is not there, or already chosen
 #pragma unroll
     for (int i = 0; i < kMine; ++i) {
         const int e = lane + i * kWave;
-        mine[i] = e < experts ? 1.0f / (1.0f + expf(-z[e])) : -1.f;  // (scores lie in [0, 1]; -1: no such expert)
+        mine[i] = e < experts ? z[e] : 0.f;  // (ranked by the logit: the score rises with it, and does not saturate)
+        if (e >= experts) out |= 1u << i;
     }
     for (int k = 0; k < top; ++k) {
-        float best = -2.f;
-        int best_e = kMaxExperts;
+        float best = 0.f;
+        int best_e = kMaxExperts;  // (none yet)
 #pragma unroll
         for (int i = 0; i < kMine; ++i) {
-            if (mine[i] > best) {  // (ascending index within the lane: the first of equals stays)
+            // (ascending index within the lane: the first of equals stays)
+            if (!((out >> i) & 1u) && (best_e == kMaxExperts || mine[i] > best)) {
                 best = mine[i];
                 best_e = lane + i * kWave;
             }
@@ -58,18 +62,19 @@ route_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
         for (int offset = kWave / 2; offset > 0; offset >>= 1) {
             const float other = __shfl_xor(best, offset, kWave);
             const int other_e = __shfl_xor(best_e, offset, kWave);
-            if (other > best || (other == best && other_e < best_e)) {
+            if (other_e != kMaxExperts &&
+                (best_e == kMaxExperts || other > best || (other == best && other_e < best_e))) {
                 best = other;
                 best_e = other_e;
             }
         }
         if (lane == 0) {
             pair_expert[static_cast<size_t>(token) * top + k] = best_e;
-            pair_weight[static_cast<size_t>(token) * top + k] = best;
+            pair_weight[static_cast<size_t>(token) * top + k] = 1.0f / (1.0f + expf(-best));
         }
 #pragma unroll
         for (int i = 0; i < kMine; ++i)
-            if (lane + i * kWave == best_e) mine[i] = -3.f;
+            if (lane + i * kWave == best_e) out |= 1u << i;
     }
 }
 
@@ -280,6 +285,7 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
 // Wave w of four owns rows 64 (w / 2) .. and the column half w % 2: 4 x 4 products of 16 x 16 per 32 k.
 constexpr int kTile = 128;
 constexpr int kSlice = 64;
+constexpr int kXcds = 8;
 
 // xs[i, :] = bf16(weight(pair) * x[token(pair), :]) for the i-th pair of the sorted order.
 __global__ void __launch_bounds__(256)
@@ -304,8 +310,20 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
                      float* __restrict__ parts, ExpertArgs a) {
     __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][kTile * kSlice];
     __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][kTile * kSlice];
-    const int tile = blockIdx.x;
-    if (tile >= *a.n_tiles) return;
+    const int K = GATE_UP ? a.hidden : a.ff;
+    const int n_out = GATE_UP ? a.ff : a.hidden;            // result columns of the expert
+    const int cols_here = GATE_UP ? kTile / 2 : kTile;      // ... of which this workgroup makes so many
+    // Workgroup b of a launch goes to XCD b % 8, and each XCD has an L2 of its own.  An XCD takes a run of
+    // neighbouring tiles (tiles are in the order of their experts) and walks it column block by column block: the
+    // workgroups that are in flight on it together share a few tiles' rows and, where neighbouring tiles are one
+    // expert's, that expert's weights.
+    const int n_tiles = *a.n_tiles;
+    const int col_blocks = (n_out + cols_here - 1) / cols_here;
+    const int per_xcd = (n_tiles + kXcds - 1) / kXcds;
+    const int turn = blockIdx.x / kXcds;
+    const int tile = (blockIdx.x % kXcds) * per_xcd + turn / col_blocks;
+    if (turn / col_blocks >= per_xcd || tile >= n_tiles) return;
+    const int c0 = (turn % col_blocks) * cols_here;
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
@@ -313,10 +331,6 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
     const int expert = a.tile_expert[tile];
     const int begin = a.tile_begin[tile];
     const int rows = a.tile_count[tile];
-    const int K = GATE_UP ? a.hidden : a.ff;
-    const int n_out = GATE_UP ? a.ff : a.hidden;            // result columns of the expert
-    const int cols_here = GATE_UP ? kTile / 2 : kTile;      // ... of which this workgroup makes so many
-    const int c0 = blockIdx.y * cols_here;
     // staging: thread t brings 16 bytes (8 k) of rows t / 8 + 32 j, j = 0..3, for A and for B
     const int s_row = threadIdx.x / 8;
     const int s_k = (threadIdx.x % 8) * 8;
@@ -499,7 +513,7 @@ CIE_API int cie_experts_gate_up(void* stream, int dtype, int mfma, const void* x
         const bf16_t* ws = static_cast<const bf16_t*>(w_gate_up);
         bf16_t* as = static_cast<bf16_t*>(act);
         if (tile_rows == kTile) {  // (x: the rows gathered in sorted order, weights applied)
-            experts_tiled_kernel<true><<<dim3(max_tiles, (ff + 63) / 64), 256, 0, s>>>(xs, ws, as, nullptr, a);
+            experts_tiled_kernel<true><<<kXcds * ((max_tiles + kXcds - 1) / kXcds) * ((ff + 63) / 64), 256, 0, s>>>(xs, ws, as, nullptr, a);
             return cie_after_launch();
         }
         if (tile_rows == 16) experts_gate_up_mfma_kernel<1><<<grid, 256, 0, s>>>(xs, ws, as, a);
@@ -535,7 +549,7 @@ CIE_API int cie_experts_down(void* stream, int dtype, int mfma, const void* act,
         const bf16_t* as = static_cast<const bf16_t*>(act);
         const bf16_t* ws = static_cast<const bf16_t*>(w_down);
         if (tile_rows == kTile) {
-            experts_tiled_kernel<false><<<dim3(max_tiles, (hidden + kTile - 1) / kTile), 256, 0, s>>>(as, ws, nullptr, parts, a);
+            experts_tiled_kernel<false><<<kXcds * ((max_tiles + kXcds - 1) / kXcds) * ((hidden + kTile - 1) / kTile), 256, 0, s>>>(as, ws, nullptr, parts, a);
             return cie_after_launch();
         }
         if (tile_rows == 16) experts_down_mfma_kernel<1><<<grid, 256, 0, s>>>(as, ws, parts, a);

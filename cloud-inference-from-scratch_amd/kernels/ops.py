@@ -1311,7 +1311,8 @@ class ExpertRoute:
 
 
 def experts_route(logits: torch.Tensor, top: int, tile_rows: int = 16) -> ExpertRoute:
-    """Scores ``sigmoid(logits)`` (float32 [T, E]), the ``top`` largest per token (lowest index first among equals),
+    """Scores ``sigmoid(logits)`` (float32 [T, E]), the ``top`` largest per token (ranked by the logits, which order
+    the scores and do not saturate; lowest index first among equals),
     and the (token, choice) pairs sorted by expert in tiles of at most ``tile_rows`` rows.  Nothing comes back to
     the host: grids are sized for ``max_tiles`` and the kernels read the true count."""
     _gpu("logits", logits, torch.float32, 2)

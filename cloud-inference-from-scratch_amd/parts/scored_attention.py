@@ -34,6 +34,7 @@ from .base import Part, register_part
 from .linear import linear
 
 _SAID_GENERIC: set = set()
+PROMPT_ROW_TILES = 4  # tiles of 16 (token, head) rows that a workgroup of the matrix-core form takes of a prompt's portion
 
 
 def _round8(n: int) -> int:
@@ -176,7 +177,7 @@ class ScoredAttention(Part):
                                                  batch.sequences, batch.seq_slot, batch.seq_start, batch.seq_q_len,
                                                  batch.q_start_loc, batch.tokens, h, g, self.kernel_dim,
                                                  self.kernel_vdim, 1, least, **shape, **shares(batch.sequences, 1))
-            row_tiles = max(least, 4 if batch.max_q_len * group > 16 else 1)
+            row_tiles = max(least, PROMPT_ROW_TILES if batch.max_q_len * group > 16 else 1)
             while row_tiles > least and -(-batch.tokens * group // (16 * row_tiles)) * g < ops.compute_units():
                 row_tiles //= 2  # (fewer rows a tile where the tiles would not fill the compute units)
             per_tile = (16 * row_tiles) // group

@@ -132,6 +132,9 @@ def make_weights(raw: dict, seed: int, sharp: float = 1.0, exact_router: bool = 
                 experts = out[name].shape[0]
                 router = torch.zeros_like(out[name])
                 router[:, : MARKERS - 1] = torch.randint(-2, 3, (experts, MARKERS - 1), generator=g).float() * 0.5
-                router[:, MARKERS - 1] = torch.arange(experts).float() / 64.0   # no two experts' logits are equal
+                # no two experts' logits are equal: the other coordinates move a logit in steps of 0.5 markers,
+                # this one by less than that in all (and stays exact in bfloat16 up to 128 experts)
+                steps = 4 << max(experts - 1, 1).bit_length()
+                router[:, MARKERS - 1] = torch.arange(experts).float() / steps
                 out[name] = router
     return {name: t.to(torch.bfloat16).float() for name, t in out.items()}

@@ -259,16 +259,25 @@ def test_a_key_is_seen_up_to_the_windows_edge_and_not_beyond(kind, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(dtype):
     """A prompt of 300 tokens, then 250 tokens decoded one by one: every window passes over decoded tokens, the
-    temperature steps many times, pages are crossed and given back.  (bfloat16: the worst of these 550 rows may lie
-    a little above the other tests' bound; the plain implementation run in bfloat16 throughout is off by 0.74 at its
-    worst row and 0.09 on average, the engine by 0.12 and 0.025.)"""
+    temperature steps many times, pages are crossed and given back.  (bfloat16: what rounding costs over 550 rows
+    is measured: the engine has to be closer to the yardstick, at its worst row and on average, than the plain
+    implementation run in bfloat16 throughout.)"""
     raw = gu.SMALL_A
     weights = gu.make_weights(raw, seed=31, exact_router=True)
     requests = {"long": random_tokens(550, raw["vocab"], 7)}
     stepper = pg.Stepper(raw, weights)
     plain = {"long": torch.cat([stepper.feed([t]) for t in requests["long"]]).float()}
     steps = replay_util.tail_one_by_one(requests, tail=250)
-    run_and_compare(raw, weights, requests, steps, dtype, plain, max_running=1, limit=0.15 if dtype == "bfloat16" else None)
+    limit = None
+    if dtype == "bfloat16":
+        rough = pg.forward(raw, weights, requests["long"], dtype=torch.bfloat16).float().numpy()
+        limit, rough_rms = gu.spread({"long": dict(enumerate(rough))}, plain)
+        assert limit < 1.0
+    runner = gu.make_runner(raw, weights, dtype, max(replay_util.max_live_tokens(steps, page=16), 16), 16, 1)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    worst, rms = gu.spread(rows, plain)
+    assert worst <= (limit or LIMIT[dtype]) and rms <= (rough_rms if limit else RMS_LIMIT[dtype]), (dtype, worst, rms)
+    assert runner.cache.stats().slots_used == 0 and runner.cache.stats().pages_used == 0
 
 
 def test_greedy_generation_through_the_engine(models):
@@ -471,6 +480,24 @@ def test_routed_experts_kernels(sizes, dtype):
     alone = ops.experts_forward(x[:1].cuda().contiguous(), ops.experts_route(logits[:1].cuda().contiguous(), top, 16),
                                 gate_up, down, 1.25, 1.702, 1.0, mfma=mfma).cpu().double()
     assert torch.equal(alone[0], parts[0])
+
+
+def test_routing_of_large_and_of_equal_logits():
+    """Logits so large that their scores round to 1 are still ranked; equal logits go to the lower index; logits of
+    minus infinity are chosen last, and with a score of zero."""
+    from cie_amd.kernels import ops
+
+    logits = torch.tensor([[20.0, 45.0, 30.0, 25.0, 45.5, -3.0],
+                           [1.0, 2.0, 2.0, 0.5, 2.0, 1.5],
+                           [float("-inf"), -100.0, float("-inf"), -95.0, float("-inf"), float("-inf")]])
+    route = ops.experts_route(logits.cuda(), 4, 16)
+    assert route.pair_expert.cpu().reshape(3, 4).tolist() == [[4, 1, 2, 3], [1, 2, 4, 5], [3, 1, 0, 2]]
+    weights = route.pair_weight.cpu().reshape(3, 4)
+    assert torch.equal(weights[0], torch.ones(4)) and torch.allclose(weights[1], torch.sigmoid(torch.tensor([2.0, 2.0, 2.0, 1.5])))
+    assert bool((weights[2] == 0).all())
+    wide = torch.zeros(2, 200)
+    wide[0, 131], wide[0, 64], wide[1, 199] = 3.0, 3.0, -1.0
+    assert ops.experts_route(wide.cuda(), 3, 16).pair_expert.cpu().reshape(2, 3).tolist() == [[64, 131, 0], [0, 1, 2]]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
