@@ -18,7 +18,7 @@ sys.path.insert(0, str(ROOT))
 WAIT_STATES = 8  # what the compiler keeps between a 16 x 16 x 32 product and a read of its sums where it counts
 
 
-def test_the_checker_sees_a_short_cut():
+def test_the_path_walk_sees_a_short_cut():
     """Pinned on a listing made by hand: straight code with enough instructions passes; a branch around them is found."""
     straight = ["v_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[4:7], a[0:3]", "s_nop 7", "v_accvgpr_read_b32 v8, a0", "s_endpgm"]
     assert mfma_hazards.short_paths(straight, WAIT_STATES) == []
