@@ -352,24 +352,41 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
         b_src[j] = weight + (static_cast<size_t>(expert) * (GATE_UP ? 2 * n_out : n_out) + col) * K;
     }
     auto place = [](int row, int piece) { return row * kSlice + ((piece ^ ((row >> 1) & 7)) << 3); };
-    uint4 ra[4], rb[4];
-    auto fetch = [&](int k0) {
-        const int k = min(k0 + s_k, K - 8);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ra[j] = *reinterpret_cast<const uint4*>(a_src[j] + k);
-            rb[j] = *reinterpret_cast<const uint4*>(b_src[j] + k);
-        }
-    };
-    auto stage = [&](int buffer, int k0) {
-        const bool k_ok = k0 + s_k < K;                         // (a slice past the end of K holds zeros on the A side)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int at = place(s_row + 32 * j, s_k >> 3);
-            *reinterpret_cast<uint4*>(&lds_a[buffer][at]) = k_ok ? ra[j] : uint4{0, 0, 0, 0};
-            *reinterpret_cast<uint4*>(&lds_b[buffer][at]) = rb[j];
-        }
-    };
+    // Two sets of registers hold the slices that are on their way: set 0 the even ones, set 1 the odd ones.  While
+    // slice s is multiplied, slices s + 1 and s + 2 are under way, so a load has two slices' products to arrive in
+    // (one was not enough: the matrix cores take a slice faster than the L2 answers under this traffic).  The sets
+    // are vector values with names of their own and the steps are macros: arrays of structs that are handed to a
+    // function by reference, or indexed by a loop's counter, went through scratch memory.
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 ra0[4], rb0[4], ra1[4], rb1[4];
+#define CIE_FETCH(fa, fb, k0_)                                                                                   \
+    {                                                                                                            \
+        const int k_ = min((k0_) + s_k, K - 8); /* (past K: clamped, and what it brings is never multiplied) */  \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                          \
+            fa[j] = *reinterpret_cast<const u32x4*>(a_src[j] + k_);                                              \
+            fb[j] = *reinterpret_cast<const u32x4*>(b_src[j] + k_);                                              \
+        }                                                                                                        \
+    }
+#define CIE_STAGE(buffer_, fa, fb, k0_)                                                                          \
+    {                                                                                                            \
+        const bool k_ok_ = (k0_) + s_k < K; /* (a slice past the end of K holds zeros on the A side) */          \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                          \
+            const int at_ = place(s_row + 32 * j, s_k >> 3);                                                     \
+            *reinterpret_cast<u32x4*>(&lds_a[buffer_][at_]) = k_ok_ ? fa[j] : u32x4{0, 0, 0, 0};                 \
+            *reinterpret_cast<u32x4*>(&lds_b[buffer_][at_]) = fb[j];                                             \
+        }                                                                                                        \
+    }
+#define CIE_MULTIPLY(buffer_)                                                                                    \
+    _Pragma("unroll") for (int half = 0; half < 2; ++half) {                                                     \
+        bf16x8 af[4], bfr[4];                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                          \
+            af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buffer_][place(row0 + i * 16 + r, half * 4 + g)]);   \
+            bfr[i] = *reinterpret_cast<const bf16x8*>(&lds_b[buffer_][place(col0 + i * 16 + r, half * 4 + g)]);  \
+        }                                                                                                        \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                            \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                        \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);          \
+    }
     floatx4 acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -377,31 +394,25 @@ experts_tiled_kernel(const bf16_t* __restrict__ a_rows, const bf16_t* __restrict
         for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     const int row0 = (wave / 2) * 64;
     const int col0 = (wave % 2) * 64;
-    fetch(0);
-    stage(0, 0);
+    CIE_FETCH(ra0, rb0, 0);
+    CIE_STAGE(0, ra0, rb0, 0);
+    CIE_FETCH(ra1, rb1, kSlice);
     __syncthreads();
-    int buffer = 0;
-    for (int k0 = 0; k0 < K; k0 += kSlice) {
-        const bool more = k0 + kSlice < K;
-        if (more) fetch(k0 + kSlice);
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            bf16x8 af[4], bfr[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buffer][place(row0 + i * 16 + r, half * 4 + g)]);
-                bfr[i] = *reinterpret_cast<const bf16x8*>(&lds_b[buffer][place(col0 + i * 16 + r, half * 4 + g)]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
-        if (more) stage(buffer ^ 1, k0 + kSlice);
+    for (int k0 = 0; k0 < K; k0 += 2 * kSlice) {
+        CIE_FETCH(ra0, rb0, k0 + 2 * kSlice);
+        CIE_MULTIPLY(0);
+        if (k0 + kSlice < K) CIE_STAGE(1, ra1, rb1, k0 + kSlice);
         __syncthreads();
-        buffer ^= 1;
+        if (k0 + kSlice < K) {
+            CIE_FETCH(ra1, rb1, k0 + 3 * kSlice);
+            CIE_MULTIPLY(1);
+            if (k0 + 2 * kSlice < K) CIE_STAGE(0, ra0, rb0, k0 + 2 * kSlice);
+            __syncthreads();
+        }
     }
+#undef CIE_FETCH
+#undef CIE_STAGE
+#undef CIE_MULTIPLY
     // lane (r, g) holds rows g*4 .. g*4+3 of row tile i at column r of column tile j
     if (GATE_UP) {
         // the wave's 64 staged columns are [gate 32 | up 32] of result columns c0 + (wave % 2) * 32 ..

@@ -444,7 +444,8 @@ def test_heads_are_normed_scaled_padded_and_cached(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(150, 8, 2, 64, 32), (7, 70, 1, 24, 40), (33, 3, 3, 50, 13), (600, 16, 4, 128, 64)])
+@pytest.mark.parametrize("sizes", [(150, 8, 2, 64, 32), (7, 70, 1, 24, 40), (33, 3, 3, 50, 13), (600, 16, 4, 128, 64),
+                                   (500, 6, 3, 328, 200)])  # (the last: several slices of k in the tiled form, and a rest)
 def test_routed_experts_kernels(sizes, dtype):
     """Choice, weights and the experts' rows against the plain functions; rows of a token do not depend on the
     tokens beside it."""
