@@ -276,7 +276,7 @@ __device__ __forceinline__ float fast_tanh(float y) {
 }
 
 template <int D, int DV, int RT>
-__global__ void __launch_bounds__(64 * kScoredWaves) scored_attention_mfma_kernel(ScoredArgs a) {
+__global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_attention_mfma_kernel(ScoredArgs a) {
     constexpr int NK = D / 32;
     constexpr int ND = DV / 16;
     constexpr int ROWS = 16 * RT;

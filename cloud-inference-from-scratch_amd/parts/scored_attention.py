@@ -34,7 +34,7 @@ from .base import Part, register_part
 from .linear import linear
 
 _SAID_GENERIC: set = set()
-PROMPT_ROW_TILES = 4  # tiles of 16 (token, head) rows that a workgroup of the matrix-core form takes of a prompt's portion
+PROMPT_ROW_TILES = 2  # tiles of 16 (token, head) rows that a workgroup of the matrix-core form takes of a prompt's portion
 
 
 def _round8(n: int) -> int:
