@@ -30,14 +30,11 @@ namespace {
 
 constexpr int kMaxExperts = 1024;
 
-// One wave per token.
-__global__ void __launch_bounds__(256)
-route_kernel(const float* __restrict__ logits, int tokens, int experts, int top, int* __restrict__ pair_expert,
-             float* __restrict__ pair_weight) {
-    const int lane = threadIdx.x % kWave;
-    const int token = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-    if (token >= tokens) return;
-    const float* z = logits + static_cast<size_t>(token) * experts;
+// One wave ranks one token's logits z: its `top` experts and their scores to expert_out / weight_out (and the
+// experts to `copy` as well, where the caller wants them in LDS).
+__device__ __forceinline__ void route_token(const float* __restrict__ z, int experts, int top, int lane,
+                                            int* __restrict__ expert_out, float* __restrict__ weight_out,
+                                            int* copy) {
     constexpr int kMine = kMaxExperts / kWave;
     float mine[kMine];
     unsigned out = 0;  // bit i: expert lane + i * kWave is not there, or already chosen
@@ -69,8 +66,9 @@ route_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
             }
         }
         if (lane == 0) {
-            pair_expert[static_cast<size_t>(token) * top + k] = best_e;
-            pair_weight[static_cast<size_t>(token) * top + k] = 1.0f / (1.0f + expf(-best));
+            expert_out[k] = best_e;
+            weight_out[k] = 1.0f / (1.0f + expf(-best));
+            if (copy) copy[k] = best_e;
         }
 #pragma unroll
         for (int i = 0; i < kMine; ++i)
@@ -78,11 +76,23 @@ route_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
     }
 }
 
+// One wave per token.
+__global__ void __launch_bounds__(256)
+route_kernel(const float* __restrict__ logits, int tokens, int experts, int top, int* __restrict__ pair_expert,
+             float* __restrict__ pair_weight) {
+    const int lane = threadIdx.x % kWave;
+    const int token = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (token >= tokens) return;
+    route_token(logits + static_cast<size_t>(token) * experts, experts, top, lane,
+                pair_expert + static_cast<size_t>(token) * top, pair_weight + static_cast<size_t>(token) * top, nullptr);
+}
+
 // One workgroup.  sorted[i]: the pair at place i of the order by expert; tiles (expert, first place, rows).
-__global__ void __launch_bounds__(1024)
-arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int tile_rows, int* __restrict__ sorted,
-               int* __restrict__ tile_expert, int* __restrict__ tile_begin, int* __restrict__ tile_count,
-               int* __restrict__ n_tiles) {
+// (pair_expert may lie in LDS.)
+__device__ __forceinline__ void arrange_pairs(const int* pair_expert, int pairs, int experts, int tile_rows,
+                                              int* __restrict__ sorted, int* __restrict__ tile_expert,
+                                              int* __restrict__ tile_begin, int* __restrict__ tile_count,
+                                              int* __restrict__ n_tiles) {
     __shared__ int count[kMaxExperts];
     __shared__ int first[kMaxExperts];
     __shared__ int first_tile[kMaxExperts];
@@ -119,6 +129,34 @@ arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int 
         const int e = pair_expert[p];
         sorted[first[e] + atomicAdd(&cursor[e], 1)] = p;
     }
+}
+
+__global__ void __launch_bounds__(1024)
+arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int tile_rows, int* __restrict__ sorted,
+               int* __restrict__ tile_expert, int* __restrict__ tile_begin, int* __restrict__ tile_count,
+               int* __restrict__ n_tiles) {
+    arrange_pairs(pair_expert, pairs, experts, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
+}
+
+// Few tokens (a step of up to sixteen single tokens): choice and order in one workgroup, one launch (beyond that
+// the waves would rank several tokens one after the other, and two launches are faster).  A wave ranks every
+// sixteenth token; the chosen experts wait in LDS for the ordering.
+constexpr int kFusedPairs = 1024;
+constexpr int kFusedTokens = 16;
+
+__global__ void __launch_bounds__(1024)
+route_arrange_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
+                     int* __restrict__ pair_expert, float* __restrict__ pair_weight, int tile_rows,
+                     int* __restrict__ sorted, int* __restrict__ tile_expert, int* __restrict__ tile_begin,
+                     int* __restrict__ tile_count, int* __restrict__ n_tiles) {
+    __shared__ int chosen[kFusedPairs];
+    const int lane = threadIdx.x % kWave;
+    for (int token = threadIdx.x / kWave; token < tokens; token += blockDim.x / kWave)
+        route_token(logits + static_cast<size_t>(token) * experts, experts, top, lane,
+                    pair_expert + static_cast<size_t>(token) * top, pair_weight + static_cast<size_t>(token) * top,
+                    chosen + token * top);
+    __syncthreads();
+    arrange_pairs(chosen, tokens * top, experts, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
 }
 
 struct ExpertArgs {
@@ -498,6 +536,11 @@ CIE_API int cie_experts_route(void* stream, const float* logits, int tokens, int
     if (tokens < 0 || experts < 1 || experts > kMaxExperts || top < 1 || top > experts || tile_rows < 1)
         return CIE_BAD_ARGUMENT;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (tokens > 0 && tokens <= kFusedTokens && tokens * top <= kFusedPairs) {
+        route_arrange_kernel<<<1, 1024, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight, tile_rows, sorted,
+                                                tile_expert, tile_begin, tile_count, n_tiles);
+        return cie_after_launch();
+    }
     if (tokens > 0) {
         route_kernel<<<(tokens + 3) / 4, 256, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight);
         if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
