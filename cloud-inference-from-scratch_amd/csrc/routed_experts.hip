@@ -191,17 +191,21 @@ __device__ __forceinline__ bf16x8 scaled_fragment(const uint4 raw, float w) {
 // under way at once, which is what a step of few rows, bound by the weights' way from memory, needs.
 constexpr int kUnroll = 4;
 
-template <int RT>
+// SPLIT: the tiles are few (a step of a few single tokens), and a wave per 16 columns would leave most SIMDs idle:
+// the workgroup's four waves share 16 columns, each takes a quarter of K, and the quarters meet in LDS, summed in
+// the waves' order.
+template <int RT, bool SPLIT>
 __global__ void __launch_bounds__(256)
 experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_gate_up,
                             bf16_t* __restrict__ act, ExpertArgs a) {
+    __shared__ float meet[SPLIT ? 3 * 2 * RT * 4 * kWave : 1];
     const int tile = blockIdx.x;
     if (tile >= *a.n_tiles) return;
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
     const int g = lane >> 4;
-    const int c0 = (blockIdx.y * 4 + wave) * 16;
+    const int c0 = SPLIT ? blockIdx.y * 16 : (blockIdx.y * 4 + wave) * 16;
     if (c0 >= a.ff) return;
     const int expert = a.tile_expert[tile];
     const int begin = a.tile_begin[tile];
@@ -222,7 +226,10 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
     floatx4 acc_g[RT], acc_u[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc_g[rt] = acc_u[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 32 * kUnroll) {
+    const int quarter = ((K + 3) / 4 + 7) & ~7;                 // (pieces of 8 k stay whole)
+    const int k_begin = SPLIT ? wave * quarter : 0;
+    const int k_end = SPLIT ? min(K, k_begin + quarter) : K;
+    for (int k0 = k_begin; k0 < k_end; k0 += 32 * kUnroll) {
         uint4 bg[kUnroll], bu[kUnroll], ax[kUnroll][RT];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -234,7 +241,7 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const bool k_ok = k0 + u * 32 + g * 8 < K;
+            const bool k_ok = k0 + u * 32 + g * 8 < k_end;
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 const bf16x8 af = scaled_fragment(ax[u][rt], k_ok ? weight[rt] : 0.f);
@@ -242,6 +249,29 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
                 acc_u[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bu[u]), acc_u[rt], 0, 0, 0);
             }
         }
+    }
+    if (SPLIT) {
+        // meet[wave - 1][gate | up][rt][i][lane]
+        if (wave > 0) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    meet[(((wave - 1) * 2 + 0) * RT + rt) * 4 * kWave + i * kWave + lane] = acc_g[rt][i];
+                    meet[(((wave - 1) * 2 + 1) * RT + rt) * 4 * kWave + i * kWave + lane] = acc_u[rt][i];
+                }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc_g[rt][i] += meet[((w * 2 + 0) * RT + rt) * 4 * kWave + i * kWave + lane];
+                    acc_u[rt][i] += meet[((w * 2 + 1) * RT + rt) * 4 * kWave + i * kWave + lane];
+                }
     }
     if (!col_ok) return;
 #pragma unroll
@@ -255,17 +285,18 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
         }
 }
 
-template <int RT>
+template <int RT, bool SPLIT>
 __global__ void __launch_bounds__(256)
 experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ w_down, float* __restrict__ parts,
                          ExpertArgs a) {
+    __shared__ float meet[SPLIT ? 3 * RT * 4 * kWave : 1];
     const int tile = blockIdx.x;
     if (tile >= *a.n_tiles) return;
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
     const int g = lane >> 4;
-    const int c0 = (blockIdx.y * 4 + wave) * 16;
+    const int c0 = SPLIT ? blockIdx.y * 16 : (blockIdx.y * 4 + wave) * 16;
     if (c0 >= a.hidden) return;
     const int expert = a.tile_expert[tile];
     const int begin = a.tile_begin[tile];
@@ -284,7 +315,10 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
     const uint4 zero = uint4{0, 0, 0, 0};
-    for (int k0 = 0; k0 < K; k0 += 32 * kUnroll) {
+    const int quarter = ((K + 3) / 4 + 7) & ~7;
+    const int k_begin = SPLIT ? wave * quarter : 0;
+    const int k_end = SPLIT ? min(K, k_begin + quarter) : K;
+    for (int k0 = k_begin; k0 < k_end; k0 += 32 * kUnroll) {
         uint4 b[kUnroll], ax[kUnroll][RT];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -295,7 +329,7 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const bool k_ok = k0 + u * 32 + g * 8 < K;
+            const bool k_ok = k0 + u * 32 + g * 8 < k_end;
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 const uint4 raw = (k_ok && row_ok[rt]) ? ax[u][rt] : zero;
@@ -303,6 +337,22 @@ experts_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restric
                                                                   __builtin_bit_cast(bf16x8, b[u]), acc[rt], 0, 0, 0);
             }
         }
+    }
+    if (SPLIT) {
+        if (wave > 0) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) meet[((wave - 1) * RT + rt) * 4 * kWave + i * kWave + lane] = acc[rt][i];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[rt][i] += meet[(w * RT + rt) * 4 * kWave + i * kWave + lane];
     }
     if (!col_ok) return;
 #pragma unroll
@@ -550,6 +600,12 @@ CIE_API int cie_experts_route(void* stream, const float* logits, int tokens, int
     return cie_after_launch();
 }
 
+// A wave per 16 result columns of every tile there can be: fewer waves than the chip has SIMDs (256 compute units of
+// four) take the form that splits K over a workgroup's waves.
+static bool few_waves(int max_tiles, int columns) {
+    return static_cast<long>(max_tiles) * ((columns + 15) / 16) <= 1024;
+}
+
 // act [pairs, ff] in the storage type, rows in sorted order.  `mfma` != 0: the matrix-core form (bfloat16, hidden
 // and ff multiples of 8, tile_rows 16 * row_tiles with row_tiles 1, 2 or 4); else tile_rows must be <= 16.
 CIE_API int cie_experts_gate_up(void* stream, int dtype, int mfma, const void* x, const void* w_gate_up, void* act,
@@ -570,9 +626,11 @@ CIE_API int cie_experts_gate_up(void* stream, int dtype, int mfma, const void* x
             experts_tiled_kernel<true><<<kXcds * ((max_tiles + kXcds - 1) / kXcds) * ((ff + 63) / 64), 256, 0, s>>>(xs, ws, as, nullptr, a);
             return cie_after_launch();
         }
-        if (tile_rows == 16) experts_gate_up_mfma_kernel<1><<<grid, 256, 0, s>>>(xs, ws, as, a);
-        else if (tile_rows == 32) experts_gate_up_mfma_kernel<2><<<grid, 256, 0, s>>>(xs, ws, as, a);
-        else if (tile_rows == 64) experts_gate_up_mfma_kernel<4><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        if (tile_rows == 16 && few_waves(max_tiles, ff))
+            experts_gate_up_mfma_kernel<1, true><<<dim3(max_tiles, (ff + 15) / 16), 256, 0, s>>>(xs, ws, as, a);
+        else if (tile_rows == 16) experts_gate_up_mfma_kernel<1, false><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        else if (tile_rows == 32) experts_gate_up_mfma_kernel<2, false><<<grid, 256, 0, s>>>(xs, ws, as, a);
+        else if (tile_rows == 64) experts_gate_up_mfma_kernel<4, false><<<grid, 256, 0, s>>>(xs, ws, as, a);
         else return CIE_BAD_ARGUMENT;
         return cie_after_launch();
     }
@@ -606,9 +664,11 @@ CIE_API int cie_experts_down(void* stream, int dtype, int mfma, const void* act,
             experts_tiled_kernel<false><<<kXcds * ((max_tiles + kXcds - 1) / kXcds) * ((hidden + kTile - 1) / kTile), 256, 0, s>>>(as, ws, nullptr, parts, a);
             return cie_after_launch();
         }
-        if (tile_rows == 16) experts_down_mfma_kernel<1><<<grid, 256, 0, s>>>(as, ws, parts, a);
-        else if (tile_rows == 32) experts_down_mfma_kernel<2><<<grid, 256, 0, s>>>(as, ws, parts, a);
-        else if (tile_rows == 64) experts_down_mfma_kernel<4><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        if (tile_rows == 16 && few_waves(max_tiles, hidden))
+            experts_down_mfma_kernel<1, true><<<dim3(max_tiles, (hidden + 15) / 16), 256, 0, s>>>(as, ws, parts, a);
+        else if (tile_rows == 16) experts_down_mfma_kernel<1, false><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        else if (tile_rows == 32) experts_down_mfma_kernel<2, false><<<grid, 256, 0, s>>>(as, ws, parts, a);
+        else if (tile_rows == 64) experts_down_mfma_kernel<4, false><<<grid, 256, 0, s>>>(as, ws, parts, a);
         else return CIE_BAD_ARGUMENT;
         return cie_after_launch();
     }
